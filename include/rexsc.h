@@ -1,0 +1,153 @@
+/*
+ * rexsc.h -- C ABI of librexsc.so: the MI355X (gfx950) implementation of REX-SC's
+ * stochastic-computing hot path.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream; no torch types.
+ * All return 0 on success and a negative code on failure; rexsc_last_error() returns the
+ * message of the calling thread's last failure.  Nothing here allocates device memory:
+ * ops that need scratch take a caller-owned workspace whose size the matching
+ * *_workspace_bytes() call reports.  Inputs are never written.  Work is enqueued on
+ * `stream` and the call returns without synchronising.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference tree, torch_c/sc-extension/ unless stated otherwise).
+ */
+#ifndef REXSC_H
+#define REXSC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *rexsc_stream_t; /* hipStream_t */
+
+enum {
+    REXSC_OK = 0,
+    REXSC_ERR_INVALID = -1,   /* bad argument / unsupported configuration */
+    REXSC_ERR_WORKSPACE = -2, /* workspace missing or too small */
+    REXSC_ERR_HIP = -3        /* a HIP runtime call failed */
+};
+
+const char *rexsc_last_error(void);
+int rexsc_version(void);
+
+/* One-time per-device set-up (LFSR sequence tables).  Called implicitly by the ops; exposed
+ * so that a caller can pay for it outside a timed or captured region. */
+int rexsc_init(rexsc_stream_t stream);
+
+/* ---- SC conv2d -------------------------------------------------------------------------
+ * Replaces sc_extension_cuda.conv2d_generic_general_split_acc / conv2d_generic_general_acc
+ * (sc_cuda.cpp:73-99) and sc_extension.conv2d_generic_general (sc_conv.cpp:301-489), with
+ * the arithmetic of the CPU extension: float operands are scaled by S (= bit_length, or
+ * 2^lfsr_length when lfsr_length > 0), clamped and ceil'ed to integers, expanded to LFSR
+ * bitstreams (XOR-feedback LFSR, seeds 1..2^lb-1), AND-multiplied, popcounted over the whole
+ * Cin*KH*KW reduction per stream cycle, clamped to n_sat per cycle and summed over cycles.
+ */
+typedef struct rexsc_conv_desc {
+    int32_t N, C, H, W;          /* activation dims, UNPADDED */
+    int32_t O, KH, KW;           /* weight dims [O][C][KH][KW] */
+    int32_t pad_h, pad_w;        /* zero padding of axis 2 / axis 3 (the reference's padding[1] / padding[0]) */
+    int32_t stride_h, stride_w;  /* stride along axis 2 / axis 3 (the reference's stride[0] / stride[1]) */
+    int32_t bit_length;          /* stream length L */
+    int32_t lfsr_length;         /* <=0: derive from L (2,4,8->3; 16->4; ... 256->8) */
+    int32_t gen_config;          /* 1 plain LFSR, 2 "and_2" generator (zero-including LFSR, 2x2 cycle interleave) */
+    int32_t bin_config;          /* n_sat = bin_config+1 if >=0 else 1-bin_config */
+    int32_t total_width, load_width, load_wait; /* progressive loading (7,8,1 = off) */
+    int32_t act_channels_last;   /* memory order of x: 0 NCHW, 1 NHWC; outputs use the same order */
+    int32_t weight_channels_last;/* memory order of w: 0 OIHW, 1 OHWI */
+} rexsc_conv_desc;
+
+size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d);
+
+/* x, w: float32 device arrays in the memory order the descriptor states.
+ * out_pos, out_neg: int16 [N][O][Ho][Wo] (or NHWC), Ho=(H+2*pad_h-KH)/stride_h+1.
+ * Either output pointer may be NULL together with out_diff != NULL to get pos-neg (int16,
+ * wrapping) instead; all three may be given. */
+int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const float *w,
+                     int16_t *out_pos, int16_t *out_neg, int16_t *out_diff,
+                     void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
+/* ---- SC linear -------------------------------------------------------------------------
+ * Replaces sc_extension_cuda.linear_generic_general_acc (sc_cuda.cpp:101-120) and
+ * sc_extension.linear_generic_general (sc_matmul.cpp:576-676).  x [B][C], w [O][C] float32
+ * row-major; out_pos/out_neg int32 [B][O].  Only the first bit_length stream slots are
+ * accumulated, and bin_config < 0 selects the "count >= n_sat" rule, as in the reference.
+ */
+typedef struct rexsc_linear_desc {
+    int32_t B, C, O;
+    int32_t bit_length, lfsr_length, gen_config, bin_config;
+    int32_t total_width, load_width, load_wait;
+} rexsc_linear_desc;
+
+size_t rexsc_linear_workspace_bytes(const rexsc_linear_desc *d);
+int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, const float *w,
+                     int32_t *out_pos, int32_t *out_neg,
+                     void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
+/* ---- OR-n pointwise activation ---------------------------------------------------------
+ * y = n - exp(-x) * sum_{i<n} (n-i) x^i / i!  for n = 1..4, float32.
+ * Replaces sc_extension_cuda.or_approx_n_forward_acc / _backward_acc (sc_cuda_pw.cu:708-811);
+ * scalar math of sc_cpu.hpp:192-262.  half_input != 0 rounds the saved pre-activation to
+ * IEEE binary16 before use, which is what the reference's backward wrapper does. */
+int rexsc_orn_forward(const float *x, float *y, size_t n, int or_n, rexsc_stream_t stream);
+int rexsc_orn_backward(const float *grad_out, const float *x, float *grad_in, size_t n, int or_n,
+                       int half_input, rexsc_stream_t stream);
+
+/* ---- fused OR-n + bias/noise error injection, both polarities --------------------------
+ * y = f(OR_n(x_pos), xi1) - f(OR_n(x_neg), xi2),  f(v, xi) = v + poly5_bias(v) + poly5_std(v)*xi,
+ * xi ~ N(0,1) from a counter-based Philox4x32-10 stream keyed by (seed, offset + element/4).
+ * Replaces sc_extension_cuda.or_approx_n_forward_bias_std_both_acc / _backward_..._both_acc
+ * (sc_cuda_pw.cu:863-927, 952-1011); scalar math of sc_cpu.hpp:264-404.
+ * bias_coef / std_coef: 6 float32 coefficients each, device memory.
+ * noise_out_pos / noise_out_neg: optional float32 [n] receiving the draws (NULL to skip). */
+int rexsc_orn_bias_std_both_forward(const float *x_pos, const float *x_neg, const float *bias_coef,
+                                    const float *std_coef, float *y, size_t n, int or_n,
+                                    uint64_t seed, uint64_t offset,
+                                    float *noise_out_pos, float *noise_out_neg, rexsc_stream_t stream);
+int rexsc_orn_bias_std_both_backward(const float *grad_out, const float *x_pos, const float *x_neg,
+                                     const float *bias_coef, float *grad_pos, float *grad_neg, size_t n,
+                                     int or_n, int half_input, rexsc_stream_t stream);
+
+/* Single-polarity variants (sc_cuda_pw.cu:834-861, 929-950).  The forward reads and writes
+ * binary16, as the reference's does. */
+int rexsc_orn_bias_std_forward_f16(const uint16_t *x_half, const float *bias_coef, const float *std_coef,
+                                   uint16_t *y_half, size_t n, int or_n, uint64_t seed, uint64_t offset,
+                                   rexsc_stream_t stream);
+int rexsc_orn_bias_std_backward(const float *grad_out, const float *x, const float *bias_coef,
+                                float *grad_in, size_t n, int or_n, int half_input, rexsc_stream_t stream);
+
+/* Philox4x32-10 block function on the host (for known-answer tests of the generator). */
+void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+
+/* ---- saturating fixed-point conv -------------------------------------------------------
+ * Replaces fixed_extension_cuda.conv2d_saturate_acc (fixed_cuda.cpp:24-34) and
+ * fixed_extension.conv2d_saturate (fixed.cpp:197-238): operands scaled by 2^precision_in,
+ * clamped, rounded half-to-even; products folded in (c, ky, kx) order through the saturating
+ * rounding adder selected by add_config (0 fixed_add, 1 fixed_add_or, >=2 pairwise OR2).
+ * x float32 NCHW [N][C][H][W], w float32 [O][C][KH][KW], out int32 NCHW = pos - neg. */
+typedef struct rexsc_fixed_desc {
+    int32_t N, C, H, W, O, KH, KW;
+    int32_t pad_h, pad_w, stride_h, stride_w;
+    int32_t add_config, precision_in, precision_out;
+} rexsc_fixed_desc;
+
+size_t rexsc_fixed_conv2d_workspace_bytes(const rexsc_fixed_desc *d);
+int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, const float *w, int32_t *out,
+                       void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
+/* ---- activation-calibration statistics -------------------------------------------------
+ * One pass over (a_bit, a_act) producing, for each of n_win (<= 64) windows
+ * win_lo[k] <= a_act < win_hi[k], the count, sum and sum of squares of err = a_bit - a_act
+ * (float64).  Windows may overlap.  Replaces the 30 masked gathers of compute_bias_std_coef
+ * (utils_functional.py:917-925).  win_lo / win_hi are HOST arrays; stats is float64
+ * [n_win][3] in device memory, zeroed by the call. */
+int rexsc_calib_stats(const float *a_bit, const float *a_act, size_t n, const float *win_lo_host,
+                      const float *win_hi_host, int n_win, double *stats, rexsc_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* REXSC_H */

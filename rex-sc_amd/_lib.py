@@ -1,0 +1,82 @@
+"""ctypes binding of librexsc.so (the C ABI declared in include/rexsc.h).
+
+The library is the only compute path: if it is missing, or an entry point fails, the caller
+gets a RuntimeError -- there is no Python/CPU fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "librexsc.so")
+_lib = None
+
+
+class ConvDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
+        "bit_length", "lfsr_length", "gen_config", "bin_config",
+        "total_width", "load_width", "load_wait", "act_channels_last", "weight_channels_last")]
+
+
+class LinearDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "B", "C", "O", "bit_length", "lfsr_length", "gen_config", "bin_config",
+        "total_width", "load_width", "load_wait")]
+
+
+class FixedDesc(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
+        "add_config", "precision_in", "precision_out")]
+
+
+_vp = ctypes.c_void_p
+_sz = ctypes.c_size_t
+_int = ctypes.c_int
+_u64 = ctypes.c_uint64
+
+# name -> (restype, argtypes); every symbol include/rexsc.h declares
+SIGNATURES = {
+    "rexsc_last_error": (ctypes.c_char_p, []),
+    "rexsc_version": (_int, []),
+    "rexsc_init": (_int, [_vp]),
+    "rexsc_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(ConvDesc)]),
+    "rexsc_conv2d_orn": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_linear_workspace_bytes": (_sz, [ctypes.POINTER(LinearDesc)]),
+    "rexsc_linear_orn": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_orn_forward": (_int, [_vp, _vp, _sz, _int, _vp]),
+    "rexsc_orn_backward": (_int, [_vp, _vp, _vp, _sz, _int, _int, _vp]),
+    "rexsc_orn_bias_std_both_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _int, _u64, _u64, _vp, _vp, _vp]),
+    "rexsc_orn_bias_std_both_backward": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _int, _int, _vp]),
+    "rexsc_orn_bias_std_forward_f16": (_int, [_vp, _vp, _vp, _vp, _sz, _int, _u64, _u64, _vp]),
+    "rexsc_orn_bias_std_backward": (_int, [_vp, _vp, _vp, _vp, _sz, _int, _int, _vp]),
+    "rexsc_philox4x32_10": (None, [ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
+                                   ctypes.POINTER(ctypes.c_uint32)]),
+    "rexsc_fixed_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(FixedDesc)]),
+    "rexsc_fixed_conv2d": (_int, [ctypes.POINTER(FixedDesc), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_calib_stats": (_int, [_vp, _vp, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float),
+                                 _int, _vp, _vp]),
+}
+
+
+def lib():
+    """Load librexsc.so once.  Raises RuntimeError if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "librexsc.so is missing (%s): build it with `python rex-sc_amd/build.py`; "
+                "there is no fallback path" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = lib().rexsc_last_error()
+        raise RuntimeError("%s failed (code %d): %s" % (what, rc, msg.decode() if msg else "?"))

@@ -1,0 +1,282 @@
+"""Tensor-level plumbing shared by the drop-in extension modules: layout decisions, workspace,
+stream, and the calls into the C ABI.  PyTorch is used for device memory and streams only."""
+import ctypes
+
+import torch
+
+import _lib
+
+# How the `xnor` argument of the conv op is treated.  The reference's CPU extension ignores it
+# (XOR-feedback LFSR, seeds 1..2^lb-1; sc_conv.cpp:362-425) while its CUDA kernels switch to an
+# XNOR LFSR.  Bit-exactness is defined against the CPU extension, so that is the only mode built.
+XNOR_MODE = "cpu_oracle"
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError("rexsc ops need tensors on a HIP device (got %s)" % t.device)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def is_channels_last(t):
+    """The reference's own layout test (sc_conv.cpp:326-331): decided from raw strides."""
+    s = t.stride()
+    return s[1] == 1 and s[1] * s[2] * s[3] != 1
+
+
+def _as_layout(t, channels_last):
+    t = t.detach()
+    if t.dtype != torch.float32:
+        t = t.float()
+    fmt = torch.channels_last if channels_last else torch.contiguous_format
+    t = t.contiguous(memory_format=fmt)
+    if channels_last and t.stride(1) != 1:  # size-1 dims make contiguous() ambiguous: force NHWC strides
+        t = t.permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)
+    if t.data_ptr() % 16:
+        t = t.clone(memory_format=torch.preserve_format)
+    return t
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def _empty_out(shape, dtype, device, channels_last):
+    if channels_last:
+        n, c, h, w = shape
+        return torch.empty((n, h, w, c), dtype=dtype, device=device).permute(0, 3, 1, 2)
+    return torch.empty(shape, dtype=dtype, device=device)
+
+
+def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
+              want_split=True, want_diff=False):
+    """SC conv2d on the HIP path.  padding=(p0,p1): p0 pads the LAST axis, p1 axis 2, as the
+    reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2."""
+    _require_cuda(x, w)
+    if x.dim() != 4 or w.dim() != 4 or x.size(1) != w.size(1):
+        raise RuntimeError("conv2d: expected input [N,C,H,W] and weight [O,C,KH,KW] with equal C, got %s and %s"
+                           % (tuple(x.shape), tuple(w.shape)))
+    cl_a, cl_w = is_channels_last(x), is_channels_last(w)
+    xc, wc = _as_layout(x, cl_a), _as_layout(w, cl_w)
+    N, C, H, W = xc.shape
+    O, _, KH, KW = wc.shape
+    d = _lib.ConvDesc(N, C, H, W, O, KH, KW, int(padding[1]), int(padding[0]), int(stride[0]), int(stride[1]),
+                      int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
+                      int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w))
+    L = _lib.lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = L.rexsc_conv2d_workspace_bytes(ctypes.byref(d))
+        if ws_bytes == 0:
+            _lib.check(-1, "rexsc_conv2d (planning)")
+        Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
+        Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
+        shape = (N, O, Ho, Wo)
+        pos = _empty_out(shape, torch.int16, x.device, cl_a) if want_split else None
+        neg = _empty_out(shape, torch.int16, x.device, cl_a) if want_split else None
+        diff = _empty_out(shape, torch.int16, x.device, cl_a) if want_diff else None
+        ws = _workspace(ws_bytes, x.device)
+        rc = L.rexsc_conv2d_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(diff),
+                                _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "rexsc_conv2d_orn")
+    return pos, neg, diff
+
+
+def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config):
+    _require_cuda(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.size(1) != w.size(1):
+        raise RuntimeError("linear: expected input [B,C] and weight [O,C], got %s and %s"
+                           % (tuple(x.shape), tuple(w.shape)))
+    xc = x.detach().float().contiguous()
+    wc = w.detach().float().contiguous()
+    B, C = xc.shape
+    O = wc.shape[0]
+    d = _lib.LinearDesc(B, C, O, int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
+                        int(prog_load[0]), int(prog_load[1]), int(prog_load[2]))
+    L = _lib.lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = L.rexsc_linear_workspace_bytes(ctypes.byref(d))
+        if ws_bytes == 0:
+            _lib.check(-1, "rexsc_linear (planning)")
+        pos = torch.empty((B, O), dtype=torch.int32, device=x.device)
+        neg = torch.empty((B, O), dtype=torch.int32, device=x.device)
+        ws = _workspace(ws_bytes, x.device)
+        rc = L.rexsc_linear_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws), ws.numel(),
+                                _stream())
+        _lib.check(rc, "rexsc_linear_orn")
+    return pos, neg
+
+
+def fixed_conv2d(x, w, add_config, precision_in, precision_out, padding, stride):
+    _require_cuda(x, w)
+    if x.dim() != 4 or w.dim() != 4 or x.size(1) != w.size(1):
+        raise RuntimeError("conv2d_saturate: expected input [N,C,H,W] and weight [O,C,KH,KW] with equal C")
+    xc, wc = _as_layout(x, False), _as_layout(w, False)  # the reference assumes NCHW (fixed.cpp:10-11)
+    N, C, H, W = xc.shape
+    O, _, KH, KW = wc.shape
+    d = _lib.FixedDesc(N, C, H, W, O, KH, KW, int(padding[1]), int(padding[0]), int(stride[0]), int(stride[1]),
+                       int(add_config), int(precision_in), int(precision_out))
+    L = _lib.lib()
+    with torch.cuda.device(x.device):
+        ws_bytes = L.rexsc_fixed_conv2d_workspace_bytes(ctypes.byref(d))
+        if ws_bytes == 0:
+            _lib.check(-1, "rexsc_fixed_conv2d (planning)")
+        Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
+        Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
+        out = torch.empty((N, O, Ho, Wo), dtype=torch.int32, device=x.device)
+        ws = _workspace(ws_bytes, x.device)
+        rc = L.rexsc_fixed_conv2d(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(out), _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "rexsc_fixed_conv2d")
+    return out
+
+
+# ---- pointwise ------------------------------------------------------------------------------
+
+def _dense_f32(t):
+    """float32, dense in memory (any permutation of a contiguous block), 16-byte aligned."""
+    t = t.detach()
+    if t.dtype != torch.float32:
+        t = t.float()
+    dense = t.is_contiguous() or (t.dim() == 4 and t.is_contiguous(memory_format=torch.channels_last))
+    if not dense:
+        t = t.contiguous()
+    if t.data_ptr() % 16:
+        t = t.clone(memory_format=torch.preserve_format)
+    return t
+
+
+def _like_layout(t, ref):
+    """float32 copy of t laid out with ref's strides (the kernels index raw storage)."""
+    t = t.detach()
+    if t.dtype != torch.float32:
+        t = t.float()
+    if t.stride() != ref.stride() or t.data_ptr() % 16:
+        out = torch.empty_like(ref)
+        out.copy_(t)
+        return out
+    return t
+
+
+def _coef(c, device):
+    c = c.detach()
+    if c.device != device or c.dtype != torch.float32 or not c.is_contiguous():
+        c = c.to(device=device, dtype=torch.float32).contiguous()
+    if c.numel() < 6:
+        raise RuntimeError("bias/std coefficient vectors need at least 6 entries (got %d)" % c.numel())
+    return c
+
+
+def orn_forward(x, or_n):
+    _require_cuda(x)
+    xf = _dense_f32(x)
+    y = torch.empty_like(xf)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().rexsc_orn_forward(_ptr(xf), _ptr(y), xf.numel(), int(or_n), _stream())
+        _lib.check(rc, "rexsc_orn_forward")
+    return y
+
+
+def orn_backward(grad_output, x, or_n, half_input=True):
+    _require_cuda(grad_output, x)
+    g = _dense_f32(grad_output)
+    xf = _like_layout(x, g)
+    gx = torch.empty_like(g)
+    with torch.cuda.device(g.device):
+        rc = _lib.lib().rexsc_orn_backward(_ptr(g), _ptr(xf), _ptr(gx), g.numel(), int(or_n), int(half_input),
+                                           _stream())
+        _lib.check(rc, "rexsc_orn_backward")
+    return gx
+
+
+_philox = {"seed": None, "offset": 0}
+
+
+def _next_philox(n_elems):
+    """(seed, offset) for the next noise draw: the seed follows torch.manual_seed, the offset
+    advances by the number of 4-element vectors consumed."""
+    seed = torch.initial_seed() & 0xFFFFFFFFFFFFFFFF
+    if _philox["seed"] != seed:
+        _philox["seed"], _philox["offset"] = seed, 0
+    off = _philox["offset"]
+    _philox["offset"] = off + (n_elems + 3) // 4
+    return seed, off
+
+
+def orn_bias_std_both_forward(x_pos, x_neg, bias_coef, std_coef, or_n, seed=None, offset=None, return_noise=False):
+    _require_cuda(x_pos, x_neg)
+    xp = _dense_f32(x_pos)
+    xn = _like_layout(x_neg, xp)
+    b, s = _coef(bias_coef, xp.device), _coef(std_coef, xp.device)
+    y = torch.empty_like(xp)
+    n = xp.numel()
+    if seed is None:
+        seed, offset = _next_philox(n)
+    np_ = torch.empty_like(xp) if return_noise else None
+    nn_ = torch.empty_like(xp) if return_noise else None
+    with torch.cuda.device(xp.device):
+        rc = _lib.lib().rexsc_orn_bias_std_both_forward(_ptr(xp), _ptr(xn), _ptr(b), _ptr(s), _ptr(y), n, int(or_n),
+                                                        int(seed), int(offset), _ptr(np_), _ptr(nn_), _stream())
+        _lib.check(rc, "rexsc_orn_bias_std_both_forward")
+    return (y, np_, nn_) if return_noise else y
+
+
+def orn_bias_std_both_backward(grad_output, x_pos, x_neg, bias_coef, or_n, half_input=True):
+    _require_cuda(grad_output, x_pos, x_neg)
+    g = _dense_f32(grad_output)
+    xp, xn = _like_layout(x_pos, g), _like_layout(x_neg, g)
+    b = _coef(bias_coef, g.device)
+    gp, gn = torch.empty_like(g), torch.empty_like(g)
+    with torch.cuda.device(g.device):
+        rc = _lib.lib().rexsc_orn_bias_std_both_backward(_ptr(g), _ptr(xp), _ptr(xn), _ptr(b), _ptr(gp), _ptr(gn),
+                                                         g.numel(), int(or_n), int(half_input), _stream())
+        _lib.check(rc, "rexsc_orn_bias_std_both_backward")
+    return gp, gn
+
+
+def orn_bias_std_forward_f16(x, bias_coef, std_coef, or_n, seed=None, offset=None):
+    _require_cuda(x)
+    xh = x.detach().to(torch.float16).contiguous()
+    b, s = _coef(bias_coef, xh.device), _coef(std_coef, xh.device)
+    y = torch.empty_like(xh)
+    if seed is None:
+        seed, offset = _next_philox(xh.numel())
+    with torch.cuda.device(xh.device):
+        rc = _lib.lib().rexsc_orn_bias_std_forward_f16(_ptr(xh), _ptr(b), _ptr(s), _ptr(y), xh.numel(), int(or_n),
+                                                       int(seed), int(offset), _stream())
+        _lib.check(rc, "rexsc_orn_bias_std_forward_f16")
+    return y
+
+
+def orn_bias_std_backward(grad_output, x, bias_coef, or_n, half_input=True):
+    _require_cuda(grad_output, x)
+    g = _dense_f32(grad_output)
+    xf = _like_layout(x, g)
+    b = _coef(bias_coef, g.device)
+    gx = torch.empty_like(g)
+    with torch.cuda.device(g.device):
+        rc = _lib.lib().rexsc_orn_bias_std_backward(_ptr(g), _ptr(xf), _ptr(b), _ptr(gx), g.numel(), int(or_n),
+                                                    int(half_input), _stream())
+        _lib.check(rc, "rexsc_orn_bias_std_backward")
+    return gx
+
+
+def calib_stats(a_bit, a_act, win_lo, win_hi):
+    """count / sum / sum-of-squares of (a_bit - a_act) per window, float64 [n_win, 3] on device."""
+    _require_cuda(a_bit, a_act)
+    ab = a_bit.detach().float().contiguous().view(-1)
+    aa = a_act.detach().float().contiguous().view(-1)
+    n_win = len(win_lo)
+    lo = (ctypes.c_float * n_win)(*[float(v) for v in win_lo])
+    hi = (ctypes.c_float * n_win)(*[float(v) for v in win_hi])
+    stats = torch.empty((n_win, 3), dtype=torch.float64, device=ab.device)
+    with torch.cuda.device(ab.device):
+        rc = _lib.lib().rexsc_calib_stats(_ptr(ab), _ptr(aa), ab.numel(), lo, hi, n_win, _ptr(stats), _stream())
+        _lib.check(rc, "rexsc_calib_stats")
+    return stats

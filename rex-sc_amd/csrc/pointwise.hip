@@ -1,0 +1,461 @@
+// OR-n pointwise activation, bias/noise error injection and calibration statistics.
+// All kernels are HBM-streaming: 128-bit loads/stores, grid sized to the chip, no LDS
+// except for the block reduction of the calibration statistics.
+//
+// Scalar math follows sc_cpu.hpp:192-404 (same fmaf order); host-side dtype conventions
+// follow sc_cuda_pw.cu:708-1011 (forward in fp32, backward on the fp16-rounded saved sum).
+#include <hip/hip_fp16.h>
+
+#include "rexsc_common.h"
+
+namespace rexsc {
+
+// ---- scalar math -------------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ float orn_fwd(float x)
+{
+    const float e = expf(-x);
+    if constexpr (N == 1) return 1.f - e;
+    if constexpr (N == 2) { float r = fmaf(-2.f, e, 2.f); return fmaf(-x, e, r); }
+    if constexpr (N == 3) {
+        const float x2 = x * x;
+        float r = fmaf(-3.f, e, 3.f);
+        r = fmaf(-2.f * x, e, r);
+        return fmaf(-0.5f * x2, e, r);
+    }
+    const float x2 = x * x;
+    float r = fmaf(-4.f, e, 4.f);
+    r = fmaf(-3.f * x, e, r);
+    const float x3 = x2 * x;
+    r = fmaf(-x2, e, r);
+    return fmaf((-1.f / 6.f) * x3, e, r);
+}
+
+// d/dx OR_n(x) * g
+template <int N>
+__device__ __forceinline__ float orn_bwd(float g, float x)
+{
+    const float e = expf(-x);
+    if constexpr (N == 1) return e * g;
+    float r = fmaf(x, e, e);
+    if constexpr (N >= 3) r = fmaf(0.5f * (x * x), e, r);
+    if constexpr (N >= 4) r = fmaf((1.f / 6.f) * ((x * x) * x), e, r);
+    return r * g;
+}
+
+struct Coef6 { float c[6]; };
+
+// The six coefficients are wave-uniform: the loads become scalar loads.
+__device__ __forceinline__ Coef6 load_coef(const float *__restrict__ p)
+{
+    Coef6 c;
+#pragma unroll
+    for (int i = 0; i < 6; i++) c.c[i] = p[i];
+    return c;
+}
+
+__device__ __forceinline__ float bias_noise_fwd(float x, float xi, const Coef6 &b, const Coef6 &s)
+{   // sc_cpu.hpp:264-284
+    const float x2 = x * x;
+    float xb = fmaf(b.c[1], x, b.c[0]);
+    const float x3 = x2 * x;
+    xb = fmaf(b.c[2], x2, xb);
+    const float x4 = x3 * x;
+    xb = fmaf(b.c[3], x3, xb);
+    const float x5 = x4 * x;
+    xb = fmaf(b.c[4], x4, xb);
+    xb = fmaf(b.c[5], x5, xb);
+    float xs = fmaf(s.c[1], x, s.c[0]);
+    xs = fmaf(s.c[2], x2, xs);
+    xs = fmaf(s.c[3], x3, xs);
+    xs = fmaf(s.c[4], x4, xs);
+    xs = fmaf(s.c[5], x5, xs);
+    return x + xb + xs * xi;
+}
+
+__device__ __forceinline__ float bias_bwd(float x, const Coef6 &b)
+{   // sc_cpu.hpp:286-297
+    const float x2 = x * x;
+    float xd = fmaf(2.f * b.c[2], x, 1.f + b.c[1]);
+    const float x3 = x2 * x;
+    xd = fmaf(3.f * b.c[3], x2, xd);
+    const float x4 = x3 * x;
+    xd = fmaf(4.f * b.c[4], x3, xd);
+    xd = fmaf(5.f * b.c[5], x4, xd);
+    return xd;
+}
+
+template <int N>
+__device__ __forceinline__ float orn_bias_bwd(float g, float x, const Coef6 &b)
+{   // sc_cpu.hpp:335-404
+    const float y = orn_fwd<N>(x);
+    const float xd = bias_bwd(y, b) * g;
+    return orn_bwd<N>(xd, x);
+}
+
+__device__ __forceinline__ float round_half(float x) { return __half2float(__float2half(x)); }
+
+// ---- Philox4x32-10 + Box-Muller ------------------------------------------------------------------
+struct U4 { uint32_t v[4]; };
+
+__host__ __device__ inline U4 philox4x32_10(U4 ctr, uint32_t k0, uint32_t k1)
+{
+    const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
+#pragma unroll
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = (uint64_t)M0 * ctr.v[0];
+        const uint64_t p1 = (uint64_t)M1 * ctr.v[2];
+        U4 n;
+        n.v[0] = (uint32_t)(p1 >> 32) ^ ctr.v[1] ^ k0;
+        n.v[1] = (uint32_t)p1;
+        n.v[2] = (uint32_t)(p0 >> 32) ^ ctr.v[3] ^ k1;
+        n.v[3] = (uint32_t)p0;
+        ctr = n;
+        k0 += W0; k1 += W1;
+    }
+    return ctr;
+}
+
+// two uniforms -> two N(0,1) draws
+__device__ __forceinline__ void box_muller(uint32_t a, uint32_t b, float &z0, float &z1)
+{
+    const float u1 = (float)((a >> 8) + 1u) * 5.9604644775390625e-8f; // (0, 1]
+    const float u2 = (float)(b >> 8) * 5.9604644775390625e-8f;        // [0, 1)
+    const float r = sqrtf(-2.f * __logf(u1));
+    z0 = r * __builtin_amdgcn_cosf(u2); // v_cos_f32 takes revolutions
+    z1 = r * __builtin_amdgcn_sinf(u2);
+}
+
+// four N(0,1) draws for vector index q of stream `which`
+__device__ __forceinline__ void normal4(uint64_t seed, uint64_t q, uint32_t which, float z[4])
+{
+    U4 ctr; ctr.v[0] = (uint32_t)q; ctr.v[1] = (uint32_t)(q >> 32); ctr.v[2] = which; ctr.v[3] = 0;
+    const U4 r = philox4x32_10(ctr, (uint32_t)seed, (uint32_t)(seed >> 32));
+    box_muller(r.v[0], r.v[1], z[0], z[1]);
+    box_muller(r.v[2], r.v[3], z[2], z[3]);
+}
+
+// ---- kernels ----------------------------------------------------------------------------------------
+constexpr int PW_THREADS = 256;
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_forward_kernel(const float *__restrict__ x, float *__restrict__ y,
+                                                                 size_t n)
+{
+    const size_t nvec = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        const float4 v = reinterpret_cast<const float4 *>(x)[q];
+        float4 r;
+        r.x = orn_fwd<N>(v.x); r.y = orn_fwd<N>(v.y); r.z = orn_fwd<N>(v.z); r.w = orn_fwd<N>(v.w);
+        reinterpret_cast<float4 *>(y)[q] = r;
+    }
+    const size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = orn_fwd<N>(x[i]);
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_backward_kernel(const float *__restrict__ g,
+                                                                  const float *__restrict__ x,
+                                                                  float *__restrict__ gx, size_t n, int half_input)
+{
+    const size_t nvec = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        float4 v = reinterpret_cast<const float4 *>(x)[q];
+        const float4 gg = reinterpret_cast<const float4 *>(g)[q];
+        if (half_input) { v.x = round_half(v.x); v.y = round_half(v.y); v.z = round_half(v.z); v.w = round_half(v.w); }
+        float4 r;
+        r.x = orn_bwd<N>(gg.x, v.x); r.y = orn_bwd<N>(gg.y, v.y); r.z = orn_bwd<N>(gg.z, v.z); r.w = orn_bwd<N>(gg.w, v.w);
+        reinterpret_cast<float4 *>(gx)[q] = r;
+    }
+    const size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) gx[i] = orn_bwd<N>(g[i], half_input ? round_half(x[i]) : x[i]);
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_bias_std_both_forward_kernel(
+    const float *__restrict__ xp, const float *__restrict__ xn, const float *__restrict__ bc, const float *__restrict__ sc,
+    float *__restrict__ y, size_t n, uint64_t seed, uint64_t offset, float *__restrict__ noise_p,
+    float *__restrict__ noise_n)
+{
+    const Coef6 b = load_coef(bc), s = load_coef(sc);
+    const size_t nvec = (n + 3) / 4; // the tail vector is handled element-wise below
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        float zp[4], zn[4];
+        normal4(seed, offset + q, 0u, zp);
+        normal4(seed, offset + q, 1u, zn);
+        if (q * 4 + 3 < n) {
+            const float4 a = reinterpret_cast<const float4 *>(xp)[q];
+            const float4 c = reinterpret_cast<const float4 *>(xn)[q];
+            float4 r;
+            r.x = bias_noise_fwd(orn_fwd<N>(a.x), zp[0], b, s) - bias_noise_fwd(orn_fwd<N>(c.x), zn[0], b, s);
+            r.y = bias_noise_fwd(orn_fwd<N>(a.y), zp[1], b, s) - bias_noise_fwd(orn_fwd<N>(c.y), zn[1], b, s);
+            r.z = bias_noise_fwd(orn_fwd<N>(a.z), zp[2], b, s) - bias_noise_fwd(orn_fwd<N>(c.z), zn[2], b, s);
+            r.w = bias_noise_fwd(orn_fwd<N>(a.w), zp[3], b, s) - bias_noise_fwd(orn_fwd<N>(c.w), zn[3], b, s);
+            reinterpret_cast<float4 *>(y)[q] = r;
+            if (noise_p) reinterpret_cast<float4 *>(noise_p)[q] = make_float4(zp[0], zp[1], zp[2], zp[3]);
+            if (noise_n) reinterpret_cast<float4 *>(noise_n)[q] = make_float4(zn[0], zn[1], zn[2], zn[3]);
+        } else {
+            for (int j = 0; j < 4; j++) {
+                const size_t i = q * 4 + j;
+                if (i >= n) break;
+                y[i] = bias_noise_fwd(orn_fwd<N>(xp[i]), zp[j], b, s) - bias_noise_fwd(orn_fwd<N>(xn[i]), zn[j], b, s);
+                if (noise_p) noise_p[i] = zp[j];
+                if (noise_n) noise_n[i] = zn[j];
+            }
+        }
+    }
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_bias_std_both_backward_kernel(
+    const float *__restrict__ g, const float *__restrict__ xp, const float *__restrict__ xn,
+    const float *__restrict__ bc, float *__restrict__ gp, float *__restrict__ gn, size_t n, int half_input)
+{
+    const Coef6 b = load_coef(bc);
+    const size_t nvec = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        float4 a = reinterpret_cast<const float4 *>(xp)[q];
+        float4 c = reinterpret_cast<const float4 *>(xn)[q];
+        const float4 gg = reinterpret_cast<const float4 *>(g)[q];
+        if (half_input) {
+            a.x = round_half(a.x); a.y = round_half(a.y); a.z = round_half(a.z); a.w = round_half(a.w);
+            c.x = round_half(c.x); c.y = round_half(c.y); c.z = round_half(c.z); c.w = round_half(c.w);
+        }
+        float4 rp, rn;
+        rp.x = orn_bias_bwd<N>(gg.x, a.x, b); rn.x = orn_bias_bwd<N>(-gg.x, c.x, b);
+        rp.y = orn_bias_bwd<N>(gg.y, a.y, b); rn.y = orn_bias_bwd<N>(-gg.y, c.y, b);
+        rp.z = orn_bias_bwd<N>(gg.z, a.z, b); rn.z = orn_bias_bwd<N>(-gg.z, c.z, b);
+        rp.w = orn_bias_bwd<N>(gg.w, a.w, b); rn.w = orn_bias_bwd<N>(-gg.w, c.w, b);
+        reinterpret_cast<float4 *>(gp)[q] = rp;
+        reinterpret_cast<float4 *>(gn)[q] = rn;
+    }
+    const size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const float a = half_input ? round_half(xp[i]) : xp[i];
+        const float c = half_input ? round_half(xn[i]) : xn[i];
+        gp[i] = orn_bias_bwd<N>(g[i], a, b);
+        gn[i] = orn_bias_bwd<N>(-g[i], c, b);
+    }
+}
+
+// single polarity, binary16 in and out (sc_cuda_pw.cu:375-418)
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_bias_std_forward_f16_kernel(const __half *__restrict__ x,
+                                                                              const float *__restrict__ bc,
+                                                                              const float *__restrict__ sc,
+                                                                              __half *__restrict__ y, size_t n,
+                                                                              uint64_t seed, uint64_t offset)
+{
+    const Coef6 b = load_coef(bc), s = load_coef(sc);
+    const size_t nvec = (n + 3) / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        float z[4];
+        normal4(seed, offset + q, 0u, z);
+        for (int j = 0; j < 4; j++) {
+            const size_t i = q * 4 + j;
+            if (i >= n) break;
+            y[i] = __float2half(bias_noise_fwd(orn_fwd<N>(__half2float(x[i])), z[j], b, s));
+        }
+    }
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_bias_std_backward_kernel(const float *__restrict__ g,
+                                                                           const float *__restrict__ x,
+                                                                           const float *__restrict__ bc,
+                                                                           float *__restrict__ gx, size_t n,
+                                                                           int half_input)
+{
+    const Coef6 b = load_coef(bc);
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        gx[i] = orn_bias_bwd<N>(g[i], half_input ? round_half(x[i]) : x[i], b);
+}
+
+// Calibration statistics: per window k, count / sum / sum of squares of (a_bit - a_act) over
+// the elements with lo[k] <= a_act < hi[k].  Windows may overlap.
+constexpr int CAL_MAX_WIN = 64;
+struct CalWindows { float lo[CAL_MAX_WIN]; float hi[CAL_MAX_WIN]; };
+
+__global__ __launch_bounds__(256) void calib_stats_kernel(const float *__restrict__ a_bit,
+                                                          const float *__restrict__ a_act, size_t n, CalWindows w,
+                                                          int n_win, double *__restrict__ stats)
+{
+    __shared__ double s_acc[CAL_MAX_WIN * 3];
+    for (int i = threadIdx.x; i < n_win * 3; i += blockDim.x) s_acc[i] = 0.0;
+    __syncthreads();
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    // Each thread keeps the sums of ONE window at a time in registers: loop windows outermost
+    // over a thread-private slice would re-read memory, so instead accumulate per element into
+    // LDS with wave-level pre-reduction.
+    for (size_t i0 = (size_t)blockIdx.x * blockDim.x; i0 < n; i0 += stride) {
+        const size_t i = i0 + threadIdx.x;
+        const bool ok = i < n;
+        const float act = ok ? a_act[i] : 0.f;
+        const float err = ok ? a_bit[i] - act : 0.f;
+        for (int k = 0; k < n_win; k++) {
+            const bool in = ok && act >= w.lo[k] && act < w.hi[k];
+            const unsigned long long m = __ballot(in);
+            if (m == 0) continue; // wave-uniform
+            double c = in ? 1.0 : 0.0, e = in ? (double)err : 0.0, e2 = in ? (double)err * (double)err : 0.0;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                c += __shfl_down(c, off);
+                e += __shfl_down(e, off);
+                e2 += __shfl_down(e2, off);
+            }
+            if ((threadIdx.x & 63) == 0) {
+                atomicAdd(&s_acc[k * 3 + 0], c);
+                atomicAdd(&s_acc[k * 3 + 1], e);
+                atomicAdd(&s_acc[k * 3 + 2], e2);
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_win * 3; i += blockDim.x)
+        if (s_acc[i] != 0.0) atomicAdd(&stats[i], s_acc[i]);
+}
+
+__global__ void zero_f64_kernel(double *p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.0;
+}
+
+// ---- host launch helpers ---------------------------------------------------------------------------
+static int pw_grid(size_t work_items)
+{
+    size_t blocks = (work_items + PW_THREADS - 1) / PW_THREADS;
+    const size_t cap = 256 * 8; // 8 blocks of 256 threads per CU
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (int)blocks;
+}
+
+#define REXSC_OR_N_SWITCH(or_n, CALL)                                      \
+    switch (or_n) {                                                        \
+    case 1: { constexpr int N = 1; CALL; } break;                          \
+    case 2: { constexpr int N = 2; CALL; } break;                          \
+    case 3: { constexpr int N = 3; CALL; } break;                          \
+    case 4: { constexpr int N = 4; CALL; } break;                          \
+    default: set_error("or_n must be 1..4 (got %d)", or_n); return REXSC_ERR_INVALID; \
+    }
+
+} // namespace rexsc
+
+using namespace rexsc;
+
+extern "C" int rexsc_orn_forward(const float *x, float *y, size_t n, int or_n, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(n == 0 || (x && y), "null pointer");
+    if (n == 0) { REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n); return REXSC_OK; }
+    const int grid = pw_grid((n + 3) / 4);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0, stream, x, y, n));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_backward(const float *g, const float *x, float *gx, size_t n, int or_n, int half_input,
+                                  rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(n == 0 || (g && x && gx), "null pointer");
+    if (n == 0) { REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n); return REXSC_OK; }
+    const int grid = pw_grid((n + 3) / 4);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0, stream, g, x,
+                                               gx, n, half_input));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_bias_std_both_forward(const float *xp, const float *xn, const float *bias_coef,
+                                               const float *std_coef, float *y, size_t n, int or_n, uint64_t seed,
+                                               uint64_t offset, float *noise_p, float *noise_n, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    REXSC_CHECK_ARG(bias_coef && std_coef && (n == 0 || (xp && xn && y)), "null pointer");
+    if (n == 0) return REXSC_OK;
+    const int grid = pw_grid((n + 3) / 4);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_both_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
+                                               stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, noise_p,
+                                               noise_n));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_bias_std_both_backward(const float *g, const float *xp, const float *xn,
+                                                const float *bias_coef, float *gp, float *gn, size_t n, int or_n,
+                                                int half_input, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    REXSC_CHECK_ARG(bias_coef && (n == 0 || (g && xp && xn && gp && gn)), "null pointer");
+    if (n == 0) return REXSC_OK;
+    const int grid = pw_grid((n + 3) / 4);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_both_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
+                                               stream, g, xp, xn, bias_coef, gp, gn, n, half_input));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_bias_std_forward_f16(const uint16_t *x_half, const float *bias_coef, const float *std_coef,
+                                              uint16_t *y_half, size_t n, int or_n, uint64_t seed, uint64_t offset,
+                                              rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    REXSC_CHECK_ARG(bias_coef && std_coef && (n == 0 || (x_half && y_half)), "null pointer");
+    if (n == 0) return REXSC_OK;
+    const int grid = pw_grid((n + 3) / 4);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_forward_f16_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
+                                               stream, reinterpret_cast<const __half *>(x_half), bias_coef, std_coef,
+                                               reinterpret_cast<__half *>(y_half), n, seed, offset));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_bias_std_backward(const float *g, const float *x, const float *bias_coef, float *gx,
+                                           size_t n, int or_n, int half_input, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    REXSC_CHECK_ARG(bias_coef && (n == 0 || (g && x && gx)), "null pointer");
+    if (n == 0) return REXSC_OK;
+    const int grid = pw_grid(n);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
+                                               stream, g, x, bias_coef, gx, n, half_input));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4])
+{
+    U4 c;
+    for (int i = 0; i < 4; i++) c.v[i] = counter[i];
+    const U4 r = philox4x32_10(c, key[0], key[1]);
+    for (int i = 0; i < 4; i++) out[i] = r.v[i];
+}
+
+extern "C" int rexsc_calib_stats(const float *a_bit, const float *a_act, size_t n, const float *starts_host,
+                                 const float *ends_host, int n_win, double *stats, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(n_win >= 1 && n_win <= CAL_MAX_WIN, "n_win must be 1..%d (got %d)", CAL_MAX_WIN, n_win);
+    REXSC_CHECK_ARG(starts_host && ends_host && stats && (n == 0 || (a_bit && a_act)), "null pointer");
+    CalWindows w;
+    for (int k = 0; k < n_win; k++) { w.lo[k] = starts_host[k]; w.hi[k] = ends_host[k]; }
+    hipLaunchKernelGGL(zero_f64_kernel, dim3(1), dim3(256), 0, stream, stats, n_win * 3);
+    REXSC_CHECK_HIP(hipGetLastError());
+    if (n == 0) return REXSC_OK;
+    const int grid = pw_grid(n);
+    hipLaunchKernelGGL(calib_stats_kernel, dim3(grid), dim3(256), 0, stream, a_bit, a_act, n, w, n_win, stats);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}

@@ -1,0 +1,300 @@
+// extern "C" entry points for SC conv2d and SC linear: validation, planning (chunk widths,
+// tiles, slot splits, workspace carving) and kernel sequencing.
+#include <stdarg.h>
+#include <string.h>
+
+#include "sc_compute.h"
+#include "sng.h"
+
+namespace rexsc {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+namespace {
+
+constexpr size_t WS_ALIGN = 256;
+// Activation streams of one batch chunk are kept below this many bytes; larger batches are
+// processed chunk by chunk with the weight streams generated once.
+constexpr size_t ACT_STREAM_CAP = (size_t)1 << 30;
+constexpr int TARGET_WAVES = 4096; // ~4 waves per SIMD on 256 CUs
+
+struct ScPlan {
+    // generators
+    GenParams gen_act, gen_w;
+    ActGeom ag;
+    WeightGeom wg;
+    // compute
+    ComputeParams cp;
+    int KW, ZC;
+    bool tuned, wide;
+    int n_chunk;       // images per batch chunk
+    int Ho, Wo;
+    // workspace (bytes)
+    size_t off_w, off_a, off_part, total;
+};
+
+int choose_zc(int Z, int KW)
+{
+    int zc = Z >= 4 ? 4 : (Z >= 2 ? 2 : 1);
+    if (KW == 1 && Z >= 8) zc = 8;
+    if (KW >= 5 && zc > 2) zc = 2;
+    return zc;
+}
+
+int fill_gen(GenParams &g, int lb, int acc, int scale, int n_slots, int div, int mul, int mod, int tw, int lw,
+             int lwait, int bit_length)
+{
+    g.lb = lb; g.acc = acc;
+    g.period = acc ? (1 << lb) : (1 << lb) - 1;
+    g.seed_mod = (1 << lb) - 1;
+    g.scale = scale;
+    g.n_slots = n_slots;
+    g.slot_div = div; g.slot_mul = mul; g.slot_mod = mod;
+    g.total_width = tw; g.load_width = lw; g.load_wait = lwait;
+    g.prog = 0;
+    REXSC_CHECK_ARG(lwait >= 1, "prog_load: load_wait must be >= 1 (got %d)", lwait);
+    for (int t = 0; t < bit_length; t++) {
+        const int sh = prog_shift(g, t);
+        REXSC_CHECK_ARG(sh >= 0 && sh < 31, "prog_load (%d,%d,%d) gives shift %d at cycle %d", tw, lw, lwait, sh, t);
+        if (sh) g.prog = 1;
+    }
+    return REXSC_OK;
+}
+
+// Common planning for conv (N images of HxW, KHxKW kernel) and linear (one "image" whose row
+// of B pixels is the batch, 1x1 kernel).
+int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int pad_h, int pad_w, int s0, int s1,
+              int bit_length, int lfsr_length, int gen_config, int bin_config, int tw, int lw, int lwait,
+              int act_cl, int w_cl, bool linear)
+{
+    memset(&pl, 0, sizeof(pl));
+    REXSC_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && O > 0 && KH > 0 && KW > 0, "non-positive dimension");
+    REXSC_CHECK_ARG(pad_h >= 0 && pad_w >= 0 && s0 > 0 && s1 > 0, "bad padding/stride");
+    REXSC_CHECK_ARG(bit_length > 0, "bit_length must be positive");
+    const int lb = lfsr_bits(bit_length, lfsr_length);
+    REXSC_CHECK_ARG(lb > 0, "unsupported stream length %d / lfsr_length %d (supported: 2,4,8,...,256 or lfsr_length 3..8)",
+                    bit_length, lfsr_length);
+    const int g = gen_config;
+    if (linear) REXSC_CHECK_ARG(g >= 1 && g <= 4, "linear: gen_config must be 1..4 (got %d)", g);
+    else REXSC_CHECK_ARG(g == 1 || g == 2, "conv2d: gen_config must be 1 (lfsr) or 2 (and_2), got %d", g);
+    const int T = bit_length * g;
+    REXSC_CHECK_ARG(bit_length <= MAX_CYCLES && T <= 4096, "stream too long (bit_length %d, gen_config %d)", bit_length, g);
+    const int scale = lfsr_length > 0 ? (1 << lfsr_length) : bit_length;
+    REXSC_CHECK_ARG(scale <= 256, "operand scale %d exceeds 8 bits", scale);
+    const int Hp = H + 2 * pad_h, Wp = W + 2 * pad_w;
+    REXSC_CHECK_ARG(Hp >= KH && Wp >= KW, "kernel larger than padded input");
+    const int Ho = (Hp - KH) / s0 + 1, Wo = (Wp - KW) / s1 + 1;
+    const int Z = ceil_div(C, 32);
+    REXSC_CHECK_ARG((long)32 * KH * KW * Z < 65536, "reduction too large: 32*KH*KW*ceil(C/32) must stay below 65536");
+
+    int n_sat = bin_config >= 0 ? bin_config + 1 : 1 - bin_config;
+    if (bin_config >= 65535) n_sat = 65535;
+    if (n_sat > 65535) n_sat = 65535;
+    const int n_slots = linear ? bit_length : T; // the linear op never visits the replicated slots
+    // 16-bit packed sums are exact for the linear op (int32 results) only while they cannot
+    // overflow; the conv op's results wrap at 16 bits in the reference as well.
+    const long per_slot_max = n_sat < 32L * KH * KW * Z ? n_sat : 32L * KH * KW * Z;
+    pl.wide = linear && bin_config >= 0 && (per_slot_max * n_slots > 65535);
+
+    pl.KW = KW; pl.Ho = Ho; pl.Wo = Wo;
+    pl.ZC = choose_zc(Z, KW);
+    if (pl.wide && pl.ZC < 4) pl.ZC = 4; // wide accumulation is built for chunk widths 4 and 8
+    pl.tuned = sc_compute_has_instance(KW, pl.ZC);
+    if (!pl.tuned) pl.ZC = Z >= 4 ? 4 : (Z >= 2 ? 2 : 1);
+    const int ZC = pl.ZC, ZG = ceil_div(Z, ZC);
+    const int OT = sc_compute_tile_ot();
+    const int O_pad = (int)align_up((size_t)O, (size_t)OT);
+    const int acc = (!linear && g == 2) ? 1 : 0;
+    int rc = fill_gen(pl.gen_act, lb, acc, scale, n_slots, g * g, g, g, tw, lw, lwait, bit_length);
+    if (rc) return rc;
+    rc = fill_gen(pl.gen_w, lb, acc, scale, n_slots, g, 1, 1, tw, lw, lwait, bit_length);
+    if (rc) return rc;
+
+    // batch chunking
+    const size_t words_per_image_slot = (size_t)ZG * Hp * Wp * ZC;
+    const size_t bytes_per_image = words_per_image_slot * n_slots * 4;
+    int n_chunk = N;
+    if (bytes_per_image * (size_t)N > ACT_STREAM_CAP) {
+        n_chunk = (int)(ACT_STREAM_CAP / bytes_per_image);
+        if (n_chunk < 1) n_chunk = 1;
+    }
+    REXSC_CHECK_ARG(words_per_image_slot * n_chunk < ((size_t)1 << 31), "activation plane too large");
+    REXSC_CHECK_ARG((long)n_chunk * Ho * Wo < (1L << 31), "too many output pixels per chunk");
+    pl.n_chunk = n_chunk;
+
+    ActGeom &ag = pl.ag;
+    ag.N = n_chunk; ag.C = C; ag.H = H; ag.W = W; ag.Hp = Hp; ag.Wp = Wp; ag.pad_h = pad_h; ag.pad_w = pad_w;
+    ag.channels_last = act_cl; ag.ZC = ZC; ag.ZG = ZG;
+    ag.slot_stride = (long)(words_per_image_slot * n_chunk);
+    if (linear) { ag.seed_cmul = 1; ag.seed_pmul = 0; }   // seed c % P + 1            (sc_matmul.cpp:302)
+    else { ag.seed_cmul = Hp * Wp; ag.seed_pmul = 1; }     // seed (c*Hp*Wp + pp) % P+1 (sc_conv.cpp:167,173)
+
+    WeightGeom &wg = pl.wg;
+    wg.O = O; wg.C = C; wg.KH = KH; wg.KW = KW; wg.channels_last = w_cl; wg.ZC = ZC; wg.ZG = ZG; wg.O_pad = O_pad;
+
+    ComputeParams &cp = pl.cp;
+    cp.M = n_chunk * Ho * Wo; cp.HoWo = Ho * Wo; cp.Wo = Wo; cp.Hp = Hp; cp.Wp = Wp; cp.s0 = s0; cp.s1 = s1;
+    cp.KH = KH; cp.ZG = ZG; cp.a_slot_stride = ag.slot_stride; cp.O = O; cp.O_pad = O_pad; cp.n_slots = n_slots;
+    cp.nn = (uint32_t)n_sat | ((uint32_t)n_sat << 16);
+    cp.mode = (linear && bin_config < 0) ? 1 : 0;
+    cp.out_channels_last = linear ? 1 : act_cl; // linear output is [B][O]
+
+    // tiling: pixels per lane and slot splits
+    const int o_tiles = O_pad / OT;
+    long waves1 = (long)ceil_div(cp.M, 256) * 4 * o_tiles;
+    cp.px = (!pl.wide && waves1 >= 2L * TARGET_WAVES) ? 2 : 1;
+    long waves = (long)ceil_div(cp.M, 256 * cp.px) * 4 * o_tiles;
+    int splits = 1;
+    if (pl.tuned && waves < TARGET_WAVES / 2) {
+        splits = (int)((TARGET_WAVES / 2 + waves - 1) / waves);
+        if (splits > n_slots) splits = n_slots;
+    }
+    cp.slots_per_split = ceil_div(n_slots, splits);
+    cp.splits = ceil_div(n_slots, cp.slots_per_split);
+    cp.direct = (!linear && cp.splits == 1 && !pl.wide) ? 1 : 0;
+    if (!pl.tuned) { cp.direct = 1; cp.splits = 1; cp.slots_per_split = n_slots; }
+
+    // workspace
+    const size_t w_bytes = (size_t)n_slots * KH * ZG * O_pad * 2 * KW * ZC * 4;
+    const size_t a_bytes = (size_t)n_slots * ag.slot_stride * 4;
+    const size_t part_bytes = cp.direct ? 0 : (size_t)(pl.wide ? 2 : 1) * cp.splits * O_pad * cp.M * 4;
+    pl.off_w = 0;
+    pl.off_a = align_up(w_bytes, WS_ALIGN);
+    pl.off_part = pl.off_a + align_up(a_bytes, WS_ALIGN);
+    pl.total = pl.off_part + align_up(part_bytes, WS_ALIGN);
+    return REXSC_OK;
+}
+
+int plan_conv(ScPlan &pl, const rexsc_conv_desc *d)
+{
+    REXSC_CHECK_ARG(d != nullptr, "null descriptor");
+    return make_plan(pl, d->N, d->C, d->H, d->W, d->O, d->KH, d->KW, d->pad_h, d->pad_w, d->stride_h, d->stride_w,
+                     d->bit_length, d->lfsr_length, d->gen_config, d->bin_config, d->total_width, d->load_width,
+                     d->load_wait, d->act_channels_last != 0, d->weight_channels_last != 0, false);
+}
+
+int plan_linear(ScPlan &pl, const rexsc_linear_desc *d)
+{
+    REXSC_CHECK_ARG(d != nullptr, "null descriptor");
+    // batch rows become the pixels of a single 1 x B "image" in channels-last order
+    int rc = make_plan(pl, 1, d->C, 1, d->B, d->O, 1, 1, 0, 0, 1, 1, d->bit_length, d->lfsr_length, d->gen_config,
+                       d->bin_config, d->total_width, d->load_width, d->load_wait, 1, 0, true);
+    if (rc) return rc;
+    if (pl.wide && !(pl.ZC == 4 || pl.ZC == 8)) {
+        set_error("linear: internal planning error (wide accumulation with chunk width %d)", pl.ZC);
+        return REXSC_ERR_INVALID;
+    }
+    return REXSC_OK;
+}
+
+} // namespace
+} // namespace rexsc
+
+using namespace rexsc;
+
+extern "C" const char *rexsc_last_error(void) { return g_error; }
+extern "C" int rexsc_version(void) { return 100; }
+
+extern "C" int rexsc_init(rexsc_stream_t stream)
+{
+    const SeqTable *t = nullptr;
+    return get_seq_tables(&t, (hipStream_t)stream);
+}
+
+extern "C" size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d)
+{
+    ScPlan pl;
+    if (plan_conv(pl, d)) return 0;
+    return pl.total;
+}
+
+extern "C" int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
+                                int16_t *out_neg, int16_t *out_diff, void *workspace, size_t workspace_bytes,
+                                rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_conv(pl, d);
+    if (rc) return rc;
+    REXSC_CHECK_ARG(x && w, "null operand pointer");
+    REXSC_CHECK_ARG(out_pos || out_neg || out_diff, "no output pointer given");
+    if (!workspace || workspace_bytes < pl.total) {
+        set_error("conv2d: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
+        return REXSC_ERR_WORKSPACE;
+    }
+    uint8_t *ws = (uint8_t *)workspace;
+    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
+    uint32_t *A = (uint32_t *)(ws + pl.off_a);
+    uint32_t *part = (uint32_t *)(ws + pl.off_part);
+
+    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, stream);
+    if (rc) return rc;
+    const size_t in_image = (size_t)d->C * d->H * d->W;
+    const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
+    for (int n0 = 0; n0 < d->N; n0 += pl.n_chunk) {
+        const int nc = d->N - n0 < pl.n_chunk ? d->N - n0 : pl.n_chunk;
+        ActGeom ag = pl.ag;
+        ComputeParams cp = pl.cp;
+        ag.N = nc;
+        cp.M = nc * pl.Ho * pl.Wo; // slot stride keeps the full-chunk value: the buffer is laid out for n_chunk images
+        rc = sng_activations(x + n0 * in_image, A, ag, pl.gen_act, stream);
+        if (rc) return rc;
+        int16_t *op = out_pos ? out_pos + n0 * out_image : nullptr;
+        int16_t *on = out_neg ? out_neg + n0 * out_image : nullptr;
+        int16_t *od = out_diff ? out_diff + n0 * out_image : nullptr;
+        if (!pl.tuned) {
+            rc = sc_compute_generic(A, Wst, cp, pl.KW, pl.ZC, op, on, od, stream);
+            if (rc) return rc;
+            continue;
+        }
+        rc = sc_compute(A, Wst, cp, pl.KW, pl.ZC, false, part, op, on, od, stream);
+        if (rc) return rc;
+        if (!cp.direct) {
+            cp.m_tiles = cp.o_tiles = 0;
+            rc = sc_finalize_i16(part, cp, op, on, od, stream);
+            if (rc) return rc;
+        }
+    }
+    return REXSC_OK;
+}
+
+extern "C" size_t rexsc_linear_workspace_bytes(const rexsc_linear_desc *d)
+{
+    ScPlan pl;
+    if (plan_linear(pl, d)) return 0;
+    return pl.total;
+}
+
+extern "C" int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, const float *w, int32_t *out_pos,
+                                int32_t *out_neg, void *workspace, size_t workspace_bytes, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_linear(pl, d);
+    if (rc) return rc;
+    REXSC_CHECK_ARG(x && w && out_pos && out_neg, "null pointer");
+    if (!workspace || workspace_bytes < pl.total) {
+        set_error("linear: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
+        return REXSC_ERR_WORKSPACE;
+    }
+    REXSC_CHECK_ARG(pl.tuned, "linear: no kernel instance for chunk width %d", pl.ZC);
+    uint8_t *ws = (uint8_t *)workspace;
+    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
+    uint32_t *A = (uint32_t *)(ws + pl.off_a);
+    uint32_t *part = (uint32_t *)(ws + pl.off_part);
+    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, stream);
+    if (rc) return rc;
+    rc = sng_activations(x, A, pl.ag, pl.gen_act, stream);
+    if (rc) return rc;
+    rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, stream);
+    if (rc) return rc;
+    return sc_finalize_i32(part, pl.cp, pl.wide, out_pos, out_neg, stream);
+}

