@@ -1,0 +1,176 @@
+#!/usr/bin/env python3
+"""Benchmark of the SC hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra]
+
+A "step" is one forward pass of all 19 stochastic-computing conv layers of ResNet-18
+(16 conv3x3 + 3 conv1x1; resnet_sc.py:33-44,246-271 of the reference) at batch 64, OR-2
+accumulation, 32-bit streams, channels_last activations, synthetic operands uniform on the
+5-bit quantisation grid -- float operands in HBM in, int16 positive/negative results in HBM out,
+i.e. exactly what sc_extension_cuda.conv2d_generic_general_split_acc does for each layer.
+The headline value is bit-MAC/s = MAC * stream length / time (one activation bit times one
+split-unipolar weight bit-pair counts as one bit-MAC).
+
+The one JSON line printed at the end also carries
+  roofline      the dominant kernel (AND/popcount compute) against the VALU integer peak:
+                achieved = algorithmic lane-ops / duration measured with HIP events on the launch
+                stream, peak = 256 CU x 64 lanes/clk x 2.4 GHz;
+  cpu_baseline  the C restatement of the reference CPU extension (oracle/, OpenMP) on a bounded
+                sample of the same workload, timed on this host;
+  extra         the other reference configurations (SC conv OR-1, SC linear fwd+bwd, fixed-point
+                conv, pointwise kernels, training steps), each with its own rate.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "rex-sc_amd"))
+
+VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9  # lane-ops/s: 256 CUs x 4 SIMD16 x 2.4 GHz
+HBM_PEAK = 8.0e12
+
+# (C_in, H_in, C_out, K, stride) for the 19 SC convs of ResNet-18 at 224x224 input
+RESNET18_SC_LAYERS = (
+    [(64, 56, 64, 3, 1)] * 4 +
+    [(64, 56, 128, 3, 2), (128, 28, 128, 3, 1), (64, 56, 128, 1, 2), (128, 28, 128, 3, 1), (128, 28, 128, 3, 1)] +
+    [(128, 28, 256, 3, 2), (256, 14, 256, 3, 1), (128, 28, 256, 1, 2), (256, 14, 256, 3, 1), (256, 14, 256, 3, 1)] +
+    [(256, 14, 512, 3, 2), (512, 7, 512, 3, 1), (256, 14, 512, 1, 2), (512, 7, 512, 3, 1), (512, 7, 512, 3, 1)]
+)
+
+
+def layer_macs(N, C, H, O, K, s):
+    Ho = (H + 2 * (K // 2) - K) // s + 1
+    return N * Ho * Ho * O * C * K * K
+
+
+def make_conv_operands(torch, N, C, H, O, K, L, seed, channels_last=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randint(0, L, (N, C, H, H), generator=g).float() / L
+    w = torch.randint(-L + 1, L, (O, C, K, K), generator=g).float() / L
+    return x, w
+
+
+def time_gpu(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--cpu-sample-batch", type=int, default=16)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the SC path has no collectives); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    import _lib
+    import sc_extension_cuda
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, OR_N, N = 32, 2, args.batch
+    _lib.check(_lib.lib().rexsc_init(None), "rexsc_init")
+
+    layers = []
+    for i, (C, H, O, K, s) in enumerate(RESNET18_SC_LAYERS):
+        x, w = make_conv_operands(torch, N, C, H, O, K, L, seed=500 + i)
+        layers.append((x.to(dev).contiguous(memory_format=torch.channels_last), w.to(dev), K, s))
+    total_mac = sum(layer_macs(N, C, H, O, K, s) for (C, H, O, K, s) in RESNET18_SC_LAYERS)
+
+    def step():
+        for (x, w, K, s) in layers:
+            sc_extension_cuda.conv2d_generic_general_split_acc(
+                x, w, L, -1, 16, (K // 2, K // 2), (s, s), (7, 8, 1), OR_N - 1, 1, True, False)
+
+    sec = time_gpu(torch, step, args.steps, args.warmup)
+    value = total_mac * L / sec
+
+    # per-kernel durations with HIP events on the launch stream (separate pass: the event
+    # bookkeeping is kept out of the headline timing)
+    _lib.profile_begin()
+    for _ in range(3):
+        step()
+    prof = _lib.profile_end()
+    comp = {k: v for k, v in prof.items() if k.startswith("sc_compute")}
+    dom_name = max(comp, key=lambda k: comp[k]["total_ms"])
+    dom = comp[dom_name]
+    achieved = dom["total_work"] / (dom["total_ms"] * 1e-3)
+    comp_ms = sum(v["total_ms"] for v in comp.values())
+    comp_ops = sum(v["total_work"] for v in comp.values())
+    roofline = {
+        "bound": "valu", "kernel": dom_name,
+        "achieved": achieved / 1e12, "peak": VALU_PEAK_LANEOPS / 1e12, "unit": "Tlane-op/s",
+        "frac": achieved / VALU_PEAK_LANEOPS, "traffic": None,
+        "avg_launch_us": dom["total_ms"] * 1e3 / dom["calls"], "launches": dom["calls"],
+        "all_compute_kernels_frac": comp_ops / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS,
+        "whole_step_frac": (total_mac * L * 4 / 32) / sec / VALU_PEAK_LANEOPS,
+        "kernel_ms_per_step": {k: round(v["total_ms"] / 3, 4) for k, v in sorted(prof.items())},
+    }
+
+    out = {
+        "metric": "sc_bit_mac_per_s", "value": value, "unit": "bit-MAC/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "resnet18_sc_conv_forward: 19 SC conv layers (16 3x3 + 3 1x1), batch %d, OR-%d, "
+                               "%d-bit streams, channels_last, float in / int16 pos+neg out" % (N, OR_N, L),
+                   "batch": N, "bit_length": L, "or_n": OR_N, "images_per_s": N / sec},
+        "roofline": roofline,
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, L, OR_N)
+    if not args.no_extra:
+        try:
+            import bench_extra
+            out["extra"] = bench_extra.run(torch, dev)
+        except Exception as e:  # the headline must survive a failure of an auxiliary config
+            out["extra"] = {"error": "%s: %s" % (type(e).__name__, e)}
+    print(json.dumps(out))
+    return 0
+
+
+def cpu_baseline(sample_batch, L, or_n):
+    """The oracle (C restatement of the reference CPU extension, OpenMP) on the same 19 layers at a
+    reduced batch; bit-MAC/s scales linearly with batch for this embarrassingly parallel op."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import oracle as orc
+    cores = orc.num_threads()
+    rng = np.random.default_rng(5)
+    mac = 0
+    t0 = time.perf_counter()
+    for (C, H, O, K, s) in RESNET18_SC_LAYERS:
+        x = (rng.integers(0, L, size=(sample_batch, C, H, H)) / L).astype(np.float32)
+        w = (rng.integers(-L + 1, L, size=(O, C, K, K)) / L).astype(np.float32)
+        orc.conv2d_generic_general_split(x, w, L, -1, 16, (K // 2, K // 2), (s, s), (7, 8, 1), or_n - 1, 1,
+                                         channels_last_activation=True)
+        mac += layer_macs(sample_batch, C, H, O, K, s)
+    sec = time.perf_counter() - t0
+    return {"value": mac * L / sec, "unit": "bit-MAC/s", "cores": cores, "kind": "port",
+            "sample": "same 19 ResNet-18 SC conv layers at batch %d (%.1f s of CPU time on %d threads)"
+                      % (sample_batch, sec, cores)}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

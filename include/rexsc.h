@@ -147,6 +147,21 @@ int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, const float *w
 int rexsc_calib_stats(const float *a_bit, const float *a_act, size_t n, const float *win_lo_host,
                       const float *win_hi_host, int n_win, double *stats, rexsc_stream_t stream);
 
+/* ---- per-kernel timing (no counterpart in the reference) --------------------------------
+ * Between rexsc_profile_begin() and rexsc_profile_end() every kernel the library launches is
+ * bracketed by two HIP events on its launch stream.  rexsc_profile_end() waits for them and
+ * returns, per kernel name, the number of launches, their summed duration and their summed
+ * algorithmic work (lane-ops for the AND/popcount kernels, bytes for the streaming kernels).
+ * Returns the number of records written (<= max_records). */
+typedef struct rexsc_profile_record {
+    char name[64];
+    int32_t calls;
+    double total_ms;
+    double total_work;
+} rexsc_profile_record;
+int rexsc_profile_begin(void);
+int rexsc_profile_end(rexsc_profile_record *out, int max_records);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,10 @@ def _p(a, typ):
     return a.ctypes.data_as(typ)
 
 
+def num_threads():
+    return int(lib().orc_num_threads())
+
+
 def lfsr_step(lb, acc, v):
     return lib().orc_lfsr_step(int(lb), int(acc), int(v))
 

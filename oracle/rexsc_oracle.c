@@ -525,3 +525,11 @@ void orc_orn_bias_std_both_backward(const float *g, const float *xp, const float
         gn[i] = orc_orn_backward_s(orc_bias_backward_s(yn, b) * (-g[i]), xn[i], or_n);
     }
 }
+
+/* Number of OpenMP threads the parallel loops above will use (for reporting). */
+#ifdef _OPENMP
+#include <omp.h>
+int orc_num_threads(void) { return omp_get_max_threads(); }
+#else
+int orc_num_threads(void) { return 1; }
+#endif

@@ -30,6 +30,11 @@ class FixedDesc(ctypes.Structure):
         "add_config", "precision_in", "precision_out")]
 
 
+class ProfileRecord(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 64), ("calls", ctypes.c_int32), ("total_ms", ctypes.c_double),
+                ("total_work", ctypes.c_double)]
+
+
 _vp = ctypes.c_void_p
 _sz = ctypes.c_size_t
 _int = ctypes.c_int
@@ -54,6 +59,8 @@ SIGNATURES = {
                                    ctypes.POINTER(ctypes.c_uint32)]),
     "rexsc_fixed_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(FixedDesc)]),
     "rexsc_fixed_conv2d": (_int, [ctypes.POINTER(FixedDesc), _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_profile_begin": (_int, []),
+    "rexsc_profile_end": (_int, [ctypes.POINTER(ProfileRecord), _int]),
     "rexsc_calib_stats": (_int, [_vp, _vp, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float),
                                  _int, _vp, _vp]),
 }
@@ -80,3 +87,15 @@ def check(rc, what):
     if rc != 0:
         msg = lib().rexsc_last_error()
         raise RuntimeError("%s failed (code %d): %s" % (what, rc, msg.decode() if msg else "?"))
+
+
+def profile_begin():
+    check(lib().rexsc_profile_begin(), "rexsc_profile_begin")
+
+
+def profile_end(max_records=64):
+    """-> {kernel name: dict(calls, total_ms, total_work)}"""
+    buf = (ProfileRecord * max_records)()
+    n = lib().rexsc_profile_end(buf, max_records)
+    return {buf[i].name.decode(): dict(calls=buf[i].calls, total_ms=buf[i].total_ms, total_work=buf[i].total_work)
+            for i in range(n)}

@@ -15,7 +15,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "librexsc.so")
-SOURCES = ["sc_api.hip", "sng.hip", "sc_compute.hip", "pointwise.hip", "fixed_conv.hip"]
+SOURCES = ["sc_api.hip", "sng.hip", "sc_compute.hip", "pointwise.hip", "fixed_conv.hip", "profile.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall", "-Wno-unused-function"]

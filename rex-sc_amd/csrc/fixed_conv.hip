@@ -9,6 +9,7 @@
 //    clamp fires it keeps firing).  This path works on int8/int16 operands quantised once.
 //  * sequential (add_config >= 1): the OR-style adders are order dependent and are evaluated
 //    product by product in the reference's (c, ky, kx) order.
+#include "profile.h"
 #include "rexsc_common.h"
 
 namespace rexsc {
@@ -199,6 +200,7 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
     REXSC_CHECK_HIP(hipGetLastError());
     const size_t nout = (size_t)p.N * p.O * p.Ho * p.Wo;
     const int grid = (int)((nout + 255) / 256 > 65536 ? 65536 : (nout + 255) / 256);
+    ProfScope prof("fixed_conv", 4.0 * nx + 4.0 * nw + 4.0 * nout, stream);
     if (p.add_config == 0) hipLaunchKernelGGL(fixed_conv_kernel<0>, dim3(grid), dim3(256), 0, stream, xq, wq, out, p);
     else if (p.add_config == 1) hipLaunchKernelGGL(fixed_conv_kernel<1>, dim3(grid), dim3(256), 0, stream, xq, wq, out, p);
     else hipLaunchKernelGGL(fixed_conv_kernel<2>, dim3(grid), dim3(256), 0, stream, xq, wq, out, p);

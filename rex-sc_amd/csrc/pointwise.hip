@@ -6,6 +6,7 @@
 // follow sc_cuda_pw.cu:708-1011 (forward in fp32, backward on the fp16-rounded saved sum).
 #include <hip/hip_fp16.h>
 
+#include "profile.h"
 #include "rexsc_common.h"
 
 namespace rexsc {
@@ -356,6 +357,7 @@ extern "C" int rexsc_orn_forward(const float *x, float *y, size_t n, int or_n, r
     REXSC_CHECK_ARG(n == 0 || (x && y), "null pointer");
     if (n == 0) { REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n); return REXSC_OK; }
     const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("orn_forward", 8.0 * n, stream);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0, stream, x, y, n));
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
@@ -368,6 +370,7 @@ extern "C" int rexsc_orn_backward(const float *g, const float *x, float *gx, siz
     REXSC_CHECK_ARG(n == 0 || (g && x && gx), "null pointer");
     if (n == 0) { REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n); return REXSC_OK; }
     const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("orn_backward", 12.0 * n, stream);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0, stream, g, x,
                                                gx, n, half_input));
     REXSC_CHECK_HIP(hipGetLastError());
@@ -383,6 +386,7 @@ extern "C" int rexsc_orn_bias_std_both_forward(const float *xp, const float *xn,
     REXSC_CHECK_ARG(bias_coef && std_coef && (n == 0 || (xp && xn && y)), "null pointer");
     if (n == 0) return REXSC_OK;
     const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("orn_bias_std_both_forward", (12.0 + (noise_p ? 4.0 : 0.0) + (noise_n ? 4.0 : 0.0)) * n, stream);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_both_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
                                                stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, noise_p,
                                                noise_n));
@@ -399,6 +403,7 @@ extern "C" int rexsc_orn_bias_std_both_backward(const float *g, const float *xp,
     REXSC_CHECK_ARG(bias_coef && (n == 0 || (g && xp && xn && gp && gn)), "null pointer");
     if (n == 0) return REXSC_OK;
     const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("orn_bias_std_both_backward", 20.0 * n, stream);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_both_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
                                                stream, g, xp, xn, bias_coef, gp, gn, n, half_input));
     REXSC_CHECK_HIP(hipGetLastError());
@@ -455,6 +460,7 @@ extern "C" int rexsc_calib_stats(const float *a_bit, const float *a_act, size_t 
     REXSC_CHECK_HIP(hipGetLastError());
     if (n == 0) return REXSC_OK;
     const int grid = pw_grid(n);
+    ProfScope prof("calib_stats", 8.0 * n, stream);
     hipLaunchKernelGGL(calib_stats_kernel, dim3(grid), dim3(256), 0, stream, a_bit, a_act, n, w, n_win, stats);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;

@@ -142,7 +142,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
 
     ComputeParams &cp = pl.cp;
     cp.M = n_chunk * Ho * Wo; cp.HoWo = Ho * Wo; cp.Wo = Wo; cp.Hp = Hp; cp.Wp = Wp; cp.s0 = s0; cp.s1 = s1;
-    cp.KH = KH; cp.ZG = ZG; cp.a_slot_stride = ag.slot_stride; cp.O = O; cp.O_pad = O_pad; cp.n_slots = n_slots;
+    cp.KH = KH; cp.ZG = ZG; cp.Z = Z; cp.a_slot_stride = ag.slot_stride; cp.O = O; cp.O_pad = O_pad; cp.n_slots = n_slots;
     cp.nn = (uint32_t)n_sat | ((uint32_t)n_sat << 16);
     cp.mode = (linear && bin_config < 0) ? 1 : 0;
     cp.out_channels_last = linear ? 1 : act_cl; // linear output is [B][O]

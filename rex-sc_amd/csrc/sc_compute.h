@@ -10,6 +10,7 @@ struct ComputeParams {
     int Hp, Wp;       // padded input plane
     int s0, s1;       // stride along h / w
     int KH, ZG;       // kernel rows, channel chunks
+    int Z;            // stream words per pixel actually carrying channels: ceil(C/32)
     long a_slot_stride; // activation words per slot
     int O, O_pad;
     int n_slots;      // slots accumulated

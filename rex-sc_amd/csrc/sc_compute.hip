@@ -14,6 +14,7 @@
 //   grid            = pixel tiles x output-channel tiles x slot splits, remapped so that the
 //                     blocks sharing a pixel tile run on the same XCD (shared L2).
 #include "sc_compute.h"
+#include "profile.h"
 
 namespace rexsc {
 
@@ -278,6 +279,10 @@ static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams 
     const long blocks = (long)p.m_tiles * p.o_tiles * p.splits;
     REXSC_CHECK_ARG(blocks < (1L << 30), "SC compute: grid too large (%ld blocks)", blocks);
     const int grid = (int)align_up((size_t)blocks, 8);
+    static char name[64] = "";
+    if (!name[0]) snprintf(name, sizeof(name), "sc_compute<%d,%d,%d,%d,%d>", KW, ZC, PX, OT, (int)WIDE);
+    // algorithmic lane-ops: (and + popcount-accumulate) x 2 polarities per 32-channel word
+    ProfScope prof(name, 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
     hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, WIDE>), dim3(grid), dim3(CB), 0, stream, A, Wst, p, part,
                        out_pos, out_neg, out_diff);
     REXSC_CHECK_HIP(hipGetLastError());
@@ -322,6 +327,7 @@ int sc_compute_generic(const uint32_t *A, const uint32_t *Wst, const ComputePara
 {
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+    ProfScope prof("sc_compute_generic", 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
     hipLaunchKernelGGL(sc_compute_generic_kernel, dim3(grid), dim3(256), 0, stream, A, Wst, p, KW, ZC, out_pos,
                        out_neg, out_diff);
     REXSC_CHECK_HIP(hipGetLastError());
@@ -333,6 +339,7 @@ int sc_finalize_i16(const uint32_t *part, const ComputeParams &p, int16_t *out_p
 {
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+    ProfScope prof("sc_finalize_i16", (double)total * (4.0 * p.splits + 4.0), stream);
     hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
                        out_neg, out_diff);
     REXSC_CHECK_HIP(hipGetLastError());
@@ -344,6 +351,7 @@ int sc_finalize_i32(const uint32_t *part, const ComputeParams &p, bool wide, int
 {
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
+    ProfScope prof("sc_finalize_i32", (double)total * (4.0 * p.splits * (wide ? 2 : 1) + 8.0), stream);
     if (wide)
         hipLaunchKernelGGL((sc_finalize_kernel<true, int32_t>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
                            out_neg, (int32_t *)nullptr);

@@ -7,6 +7,7 @@
 // Semantics follow the reference CPU extension: sc_conv.cpp:42-200 (conv), sc_matmul.cpp:3-383
 // (linear); quantisation sc_conv.cpp:316-320.
 #include "sng.h"
+#include "profile.h"
 
 namespace rexsc {
 
@@ -254,6 +255,9 @@ static int launch_act(const float *x, uint32_t *A, const SeqTable *tables, const
                       hipStream_t stream)
 {
     dim3 grid(ceil_div(geo.Hp * geo.Wp, ACT_TILE), geo.ZG, geo.N);
+    // algorithmic bytes: fp32 operands in, stream words out
+    ProfScope prof("sng_act", 4.0 * geo.N * geo.C * geo.H * geo.W + 4.0 * gp.n_slots * geo.N * geo.ZG * geo.Hp * geo.Wp * ZC,
+                   stream);
     hipLaunchKernelGGL(sng_act_kernel<ZC>, grid, dim3(256), 0, stream, x, A, tables, geo, gp);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
@@ -284,6 +288,8 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
     if (slot_group > W_SLOT_GROUP) slot_group = W_SLOT_GROUP;
     REXSC_CHECK_ARG(slot_group >= 1, "weight SNG: kernel width %d too large for LDS staging", geo.KW);
     const size_t lds = SEQ_LEN + 256 + row_bytes * slot_group;
+    ProfScope prof("sng_weight", 4.0 * geo.O * geo.C * geo.KH * geo.KW +
+                                     4.0 * gp.n_slots * geo.KH * geo.ZG * geo.O_pad * 2 * geo.KW * ZC, stream);
     hipLaunchKernelGGL(sng_weight_kernel<ZC>, grid, dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
