@@ -1,0 +1,371 @@
+"""Host-side counterpart of the reference's utils_functional.py for the SC hot path.
+
+Same names and argument meaning as the reference (quantize / QuantizeGrad :93-123, the
+autograd wrappers :468-587, compute_bias_std_coef :900-949, conv2d_generic :1083-1317), live
+branches only, calling the drop-in extension modules of this package.  What "backward" means
+is unchanged: autograd runs through a float surrogate (F.conv2d on the positive / negative
+weight parts followed by the OR-n closed form); the integer SC result only replaces the
+surrogate's forward values.
+"""
+import math
+import os
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import _ops
+import fixed_extension_cuda
+import sc_extension_cuda
+
+prec_default = 7      # utils_functional.py:31
+LFSR_Length = -1      # :44  always the maximal-length LFSR of the stream length
+XNOR = True           # :45  passed through; the op follows the CPU extension and ignores it
+MUX = False           # :46
+Use_Approx = False    # config.py
+
+
+# ---- small helpers (utils_functional.py:52-91) ----------------------------------------------
+def setattr_default(obj, kwargs, att_string, default_value):
+    if att_string in kwargs:
+        setattr(obj, att_string, kwargs.pop(att_string))
+    else:
+        setattr(obj, att_string, default_value)
+
+
+def setdict_default(d, kwargs, att_string, default_value):
+    d[att_string] = kwargs.pop(att_string) if att_string in kwargs else default_value
+
+
+def setvalue_default(kwargs, att_string, default_value):
+    return kwargs.pop(att_string) if att_string in kwargs else default_value
+
+
+def update_sync(model, sync=1):
+    for mod in model.modules():
+        if isinstance(mod, (nn.Conv2d, nn.Linear)) and hasattr(mod, "run_args"):
+            mod.run_args["sync"] = sync
+
+
+def quantize(input, prec=8):
+    """(x * 2^prec).round().clamp(+-(2^prec - 1)) / 2^prec  (utils_functional.py:93-104, prune = 0)."""
+    if prec <= 16:
+        prec_2 = 2 ** prec
+        return (input * prec_2).round().clamp(-prec_2 + 1, prec_2 - 1) / prec_2
+    return input.clamp(-1, 1)
+
+
+class QuantizeGrad(torch.autograd.Function):
+    """Quantise forward, straight-through backward (utils_functional.py:117-123)."""
+
+    @staticmethod
+    def forward(ctx, x, prec):
+        return quantize(x, prec=prec)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        return grad_output, None
+
+
+# ---- OR-n activation and error injection -------------------------------------------------------
+def _orn_torch_forward(s, n):
+    # utils_functional.py:476-482 (n > 4: no fused kernel)
+    e = torch.exp(-s)
+    out = n
+    for i in range(n):
+        out = out - (n - i) * (s ** i) * (1 / math.factorial(i)) * e
+    return out
+
+
+def _orn_torch_backward(g, s, n):
+    # utils_functional.py:491-495
+    e = torch.exp(-s)
+    gi = 0
+    for i in range(n):
+        gi = gi + (1 / math.factorial(i)) * (s ** i) * e
+    return gi * g
+
+
+class Or_Approx_n_Grad(torch.autograd.Function):
+    """y = OR_n(sum); only `sum` is saved (utils_functional.py:468-495)."""
+
+    @staticmethod
+    def forward(ctx, sum, n):
+        ctx.n = n
+        ctx.save_for_backward(sum)
+        if n <= 4:
+            return sc_extension_cuda.or_approx_n_forward_acc(sum, n)
+        return _orn_torch_forward(sum, n)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        n = ctx.n
+        sum, = ctx.saved_tensors
+        if n <= 4:
+            return sc_extension_cuda.or_approx_n_backward_acc(grad_output, sum, n), None
+        return _orn_torch_backward(grad_output, sum, n), None
+
+
+class Or_Approx_N_Bias_Correct_Grad_Both(torch.autograd.Function):
+    """Fused OR_n + bias/noise injection on both polarities and their difference
+    (utils_functional.py:559-575)."""
+
+    @staticmethod
+    def forward(ctx, sum_pos, sum_neg, n, bias_coef, std_coef, order):
+        ctx.n = n
+        ctx.order = order
+        ctx.save_for_backward(sum_pos, sum_neg, bias_coef)
+        return sc_extension_cuda.or_approx_n_forward_bias_std_both_acc(sum_pos, sum_neg, bias_coef, std_coef, n)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        sum_pos, sum_neg, bias_coef = ctx.saved_tensors
+        gp, gn = sc_extension_cuda.or_approx_n_backward_bias_std_both_acc(grad_output, sum_pos, sum_neg, bias_coef,
+                                                                           ctx.n)
+        return gp, gn, None, None, None, None
+
+
+def _poly5(c, x):
+    return c[0] + c[1] * x + c[2] * x ** 2 + c[3] * x ** 3 + c[4] * x ** 4 + c[5] * x ** 5
+
+
+class Bias_Correct_Grad(torch.autograd.Function):
+    """x + poly_bias(x) + poly_std(x) * N(0,1) (utils_functional.py:441-459, 577-587).  Used only at
+    calibration steps, so it stays on plain torch ops."""
+
+    @staticmethod
+    def forward(ctx, x, bias_coef, std_coef, order):
+        ctx.order = order
+        ctx.save_for_backward(x, bias_coef)
+        x_with_rand = x + _poly5(std_coef, x) * torch.randn_like(x)
+        return x_with_rand + _poly5(bias_coef, x)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, b = ctx.saved_tensors
+        x_dot = 1 + b[1] + b[2] * 2 * x + b[3] * 3 * x ** 2 + b[4] * 4 * x ** 3 + b[5] * 5 * x ** 4
+        return x_dot * grad_output, None, None, None
+
+
+def or_approx_no(sum, n):
+    """OR-n keeping only the n-th bit (utils_functional.py:590-598)."""
+    e = torch.exp(-sum)
+    out = 1
+    for i in range(n):
+        out = out - (sum ** i) * (1 / math.factorial(i)) * e
+    return out
+
+
+def or_approx_2_1(sum, n):
+    return (sum / n) ** n + ((sum / n) ** (n - 1)) * (1 - sum / n) * n
+
+
+def or_approx_2_4(sum, n):
+    return 1 - torch.exp(-sum) + (sum / n) ** n
+
+
+# ---- calibration -----------------------------------------------------------------------------
+CALIB_WINDOWS = 30
+CALIB_WIDTH = 0.1
+
+
+def compute_bias_std_coef(or_n, a_bit, a_act, order):
+    """Fit the bias / std polynomials of the SC error (utils_functional.py:900-949).
+
+    Windows [s, s+0.1) with s on linspace(0, max(a_bit), 30) are selected on the float surrogate
+    a_act; each window with more than one sample contributes the mean and the unbiased std of
+    a_bit - a_act.  The reference gathers every window with a boolean mask (60 passes over the
+    tensors); here one kernel accumulates count / sum / sum of squares for all windows and the
+    two 30 x (order+1) least-squares problems are solved on the host in float64.
+    """
+    if int(os.environ.get("Weight_Prec", "-1")) > 0:
+        or_n = 1
+    dev = a_bit.device
+    if or_n < 0:
+        return torch.zeros(order + 1, device=dev), torch.zeros(order + 1, device=dev)
+    output_range = np.linspace(0, a_bit.max().item(), CALIB_WINDOWS)
+    lo = [np.float32(s) for s in output_range]
+    hi = [np.float32(s + CALIB_WIDTH) for s in output_range]
+    stats = _ops.calib_stats(a_bit.reshape(-1), a_act.reshape(-1), lo, hi).cpu().numpy()
+    cnt, s1, s2 = stats[:, 0], stats[:, 1], stats[:, 2]
+    valid = np.nonzero(cnt > 1)[0]
+    n = cnt[valid]
+    mean = s1[valid] / n
+    var = np.maximum(s2[valid] - s1[valid] * s1[valid] / n, 0.0) / (n - 1)
+    bias_bins = mean.astype(np.float32)
+    std_bins = np.sqrt(var).astype(np.float32)
+    pos = output_range[valid]
+    A = np.stack([pos ** i for i in range(order + 1)], axis=1).astype(np.float32).astype(np.float64)
+    if order >= len(valid) // 5:
+        bias_coef = np.zeros(order + 1, np.float32)
+    else:
+        bias_coef = np.linalg.lstsq(A, bias_bins.astype(np.float64), rcond=None)[0].astype(np.float32)
+    if len(valid) == 0:
+        std_coef = np.zeros(order + 1, np.float32)
+    else:
+        std_coef = np.linalg.lstsq(A, std_bins.astype(np.float64), rcond=None)[0].astype(np.float32)
+    return torch.from_numpy(bias_coef).to(dev), torch.from_numpy(std_coef).to(dev)
+
+
+# ---- generic SC layers ------------------------------------------------------------------------
+def _parse_forward(forward, generator):
+    """forward / generator strings -> (or_n, bin_config, gen_config) (utils_functional.py:1160-1178)."""
+    or_n, bin_config = -1, None
+    if forward[:3] == "or_":
+        if len(forward) == 4:
+            or_n = int(forward[-1]); bin_config = or_n - 1
+        elif len(forward) == 5:
+            or_n = int(forward[3]); bin_config = -or_n + 1
+        elif len(forward) == 6:
+            or_n = int(forward[-1]); bin_config = or_n
+    elif forward == "full_or":
+        bin_config = 0
+    elif forward == "full_bin":
+        bin_config = 51200
+    gen_config = None
+    if generator in ("lfsr", "lfsr_mult", "lfsr_split"):
+        gen_config = 1
+    elif generator[:4] == "and_":
+        gen_config = int(generator[-1])
+    return or_n, bin_config, gen_config
+
+
+def conv2d_generic(activation, weight, padding, stride, **kwargs):
+    """Generic SC conv2d (utils_functional.py:1083-1317).
+
+    sync = 1: SC forward (integer kernels) over the OR-n float surrogate;
+    sync = 2: as 1, plus calibration of the bias/std polynomials (returns them as well);
+    sync = 3: no SC kernels, fused OR-n + bias/noise error injection on the surrogate;
+    sync = 0: surrogate only.
+    padding[0] pads the last axis and padding[1] axis 2, as the reference's F.pad call does.
+    """
+    bit_length = setvalue_default(kwargs, "bit_length", 128)
+    generator = setvalue_default(kwargs, "generator", None)
+    forward = setvalue_default(kwargs, "forward", "full_or")
+    load_unit = setvalue_default(kwargs, "load_unit", 8)
+    load_wait_w = setvalue_default(kwargs, "load_wait_w", 1)
+    split_output = setvalue_default(kwargs, "split_output", False)
+    order = setvalue_default(kwargs, "order", 10)
+    z_unit = setvalue_default(kwargs, "z_unit", 16)
+    bias_coef = setvalue_default(kwargs, "bias_coef", None)
+    std_coef = setvalue_default(kwargs, "std_coef", None)
+    sync_override = setvalue_default(kwargs, "sync", 1)
+    if bias_coef is None:
+        bias_coef = torch.zeros(order + 1, device=activation.device)
+    if std_coef is None:
+        std_coef = torch.zeros(order + 1, device=activation.device)
+    if generator is None:
+        raise ValueError("conv2d_generic: a generator must be given ('lfsr', 'and_2', 'fixed')")
+
+    dtype = torch.float16 if torch.is_autocast_enabled() else activation.dtype
+    pad_hw = (int(padding[1]), int(padding[0]))  # (axis 2, axis 3) for F.conv2d
+    or_n, bin_config, gen_config = _parse_forward(forward, generator)
+    global_sync = os.environ.get("Global_Sync", "1") == "1"
+    sc_on = global_sync and (not Use_Approx) and 0 < sync_override < 3
+
+    result_pos = result_neg = None
+    if sc_on:
+        with torch.no_grad():
+            if bin_config is not None and gen_config is not None:
+                result_pos, result_neg = sc_extension_cuda.conv2d_generic_general_split_acc(
+                    activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
+                    (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
+                result_pos = result_pos.to(dtype=dtype)
+                result_neg = result_neg.to(dtype=dtype)
+            if generator == "fixed":
+                result_pos = fixed_extension_cuda.conv2d_saturate_acc(
+                    activation.data, weight.data, 0, int(np.log2(bit_length)), 24, padding, stride).to(dtype=dtype)
+                result_neg = torch.zeros_like(result_pos)
+                result_pos = result_pos / bit_length
+                result_neg = result_neg / bit_length
+            if result_pos is None:
+                raise ValueError("conv2d_generic: no SC kernel for forward=%r with generator=%r" % (forward, generator))
+
+    w_pos = weight.clamp(0, 100)
+    w_neg = -(weight.clamp(-100, 0))
+    activation = activation.to(w_pos.dtype)
+
+    if sync_override >= 0:
+        if forward in ("full_or", "and_2"):
+            result_pos_value = Or_Approx_n_Grad.apply(F.conv2d(activation, w_pos, padding=pad_hw, stride=stride), 1)
+            result_neg_value = Or_Approx_n_Grad.apply(F.conv2d(activation, w_neg, padding=pad_hw, stride=stride), 1)
+        elif forward[:3] == "or_":
+            conv_pos_normal = F.conv2d(activation, w_pos, padding=pad_hw, stride=stride)
+            conv_neg_normal = F.conv2d(activation, w_neg, padding=pad_hw, stride=stride)
+            if len(forward) == 4:
+                if sync_override == 3:
+                    return Or_Approx_N_Bias_Correct_Grad_Both.apply(conv_pos_normal, conv_neg_normal, or_n, bias_coef,
+                                                                    std_coef, order).to(dtype)
+                result_pos_value = Or_Approx_n_Grad.apply(conv_pos_normal, or_n)
+                result_neg_value = Or_Approx_n_Grad.apply(conv_neg_normal, or_n)
+            elif len(forward) == 5:
+                result_pos_value = or_approx_no(conv_pos_normal, or_n)
+                result_neg_value = or_approx_no(conv_neg_normal, or_n)
+            else:
+                k = weight.size(1) * weight.size(2) * weight.size(3)
+                fn = or_approx_2_1 if int(forward[-1]) == 1 else or_approx_2_4
+                result_pos_value = fn(conv_pos_normal, k)
+                result_neg_value = fn(conv_neg_normal, k)
+        elif forward == "full_bin":
+            result_pos_value = F.conv2d(activation, weight.clamp(-100, 100), padding=pad_hw, stride=stride)
+            result_neg_value = torch.zeros_like(result_pos_value)
+        else:
+            raise ValueError("conv2d_generic: unknown forward %r" % forward)
+    else:
+        raise ValueError("conv2d_generic: sync must be >= 0")
+
+    if sc_on and sync_override == 1:
+        # the SC result replaces the float forward; gradients still flow through the surrogate
+        result_pos_value.data = result_pos / bit_length
+        result_neg_value.data = result_neg / bit_length
+    elif sync_override == 2:
+        with torch.no_grad():
+            result_bit = torch.cat([(result_pos / bit_length).reshape(-1), (result_neg / bit_length).reshape(-1)])
+            result_act = torch.cat([result_pos_value.reshape(-1), result_neg_value.reshape(-1)])
+            bias_coef_new, std_coef_new = compute_bias_std_coef(or_n, result_bit, result_act, order)
+            bias_coef[:bias_coef_new.size(0)] = bias_coef_new
+            std_coef[:std_coef_new.size(0)] = std_coef_new
+        result_pos_value = Bias_Correct_Grad.apply(result_pos_value, bias_coef, std_coef, order)
+        result_neg_value = Bias_Correct_Grad.apply(result_neg_value, bias_coef, std_coef, order)
+
+    result_pos_value.data = result_pos_value.data.to(dtype)
+    result_neg_value.data = result_neg_value.data.to(dtype)
+    if split_output:
+        return result_pos_value, result_neg_value
+    if sync_override == 2:
+        return result_pos_value - result_neg_value, bias_coef, std_coef
+    return result_pos_value - result_neg_value
+
+
+def linear_generic_sc(activation, weight, **kwargs):
+    """SC linear layer on the extension's semantics (sc_matmul.cpp:576-676): integer SC forward over
+    the float surrogate OR_n(x w_pos^T) - OR_n(x w_neg^T).  (The reference's own `linear_generic`
+    is a legacy pure-torch simulation with different seeds and never calls the extension.)"""
+    bit_length = setvalue_default(kwargs, "bit_length", 128)
+    forward = setvalue_default(kwargs, "forward", "or_2")
+    generator = setvalue_default(kwargs, "generator", "lfsr")
+    load_unit = setvalue_default(kwargs, "load_unit", 8)
+    load_wait_w = setvalue_default(kwargs, "load_wait_w", 1)
+    sync_override = setvalue_default(kwargs, "sync", 1)
+    or_n, bin_config, gen_config = _parse_forward(forward, generator)
+    if bin_config is None or gen_config is None:
+        raise ValueError("linear_generic_sc: unsupported forward=%r / generator=%r" % (forward, generator))
+    w_pos = weight.clamp(0, 100)
+    w_neg = -(weight.clamp(-100, 0))
+    lin_pos = F.linear(activation, w_pos)
+    lin_neg = F.linear(activation, w_neg)
+    if forward == "full_bin":
+        pos_value, neg_value = lin_pos, lin_neg
+    else:
+        n = or_n if or_n > 0 else 1
+        pos_value = Or_Approx_n_Grad.apply(lin_pos, n)
+        neg_value = Or_Approx_n_Grad.apply(lin_neg, n)
+    if sync_override == 1:
+        with torch.no_grad():
+            pos, neg = sc_extension_cuda.linear_generic_general_acc(
+                activation.data, weight.data, (prec_default, load_unit, load_wait_w), bit_length, LFSR_Length,
+                bin_config, gen_config, XNOR, MUX)
+        pos_value.data = pos.to(activation.dtype) / bit_length
+        neg_value.data = neg.to(activation.dtype) / bit_length
+    return pos_value - neg_value

@@ -1,0 +1,190 @@
+"""What the mathematics fixes about the oracle, independent of the golden vectors: LFSR cycle
+structure, stream density, special cases that reduce to library routines, closed forms."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle as orc
+
+
+@pytest.mark.parametrize("lb", [3, 4, 5, 6, 7, 8])
+def test_lfsr_is_maximal_length(lb):
+    period = (1 << lb) - 1
+    seen, v = [], 1
+    for _ in range(period):
+        seen.append(v)
+        v = orc.lfsr_step(lb, 0, v)
+    assert v == 1 and sorted(seen) == list(range(1, period + 1))
+    assert orc.lfsr_step(lb, 0, 0) == 0  # zero is a fixed point of the plain LFSR
+    # the zero-including flavour visits all 2^lb states
+    seen, v = [], 1
+    for _ in range(1 << lb):
+        seen.append(v)
+        v = orc.lfsr_step(lb, 1, v)
+    assert v == 1 and sorted(seen) == list(range(1 << lb))
+
+
+def test_lfsr_bits_fall_through():
+    assert [orc.lfsr_bits(b) for b in (2, 4, 8, 16, 32, 64, 128, 256)] == [3, 3, 3, 4, 5, 6, 7, 8]
+    assert orc.lfsr_bits(48) == -1 and orc.lfsr_bits(32, 7) == 7
+
+
+def test_quantize_closed_forms():
+    x = np.array([-0.5, 0.0, 1 / 64, 1 / 32, 0.51, 31 / 32, 1.0, 2.0], np.float32)
+    assert orc.quantize_sc(x, 32, 0).tolist() == [0, 0, 1, 1, 17, 31, 31, 31]
+    assert orc.quantize_sc(-x, 32, 1).tolist() == [0, 0, 1, 1, 17, 31, 31, 31]
+    assert orc.quantize_sc(x, 32, 1).tolist() == [16, 0, 0, 0, 0, 0, 0, 0]
+    h = np.array([0.5 / 32, 1.5 / 32, 2.5 / 32, 0.49 / 32], np.float32)
+    assert orc.quantize_fixed(h, 32, 0).tolist() == [0, 2, 2, 0]  # half to even
+
+
+def test_single_element_stream_density():
+    """One activation against weight 1-1/L: over the L cycles a value v gives v or v-1 ones (the
+    LFSR visits every state 1..L-1 once, and one of them twice)."""
+    L = 32
+    for v in range(L):
+        x = np.full((1, 1, 1, 1), v / L, np.float32)
+        w = np.full((1, 1, 1, 1), 1.0, np.float32)  # quantises to L-1: its stream is 1 except where state == L-1
+        pos, neg = orc.conv2d_generic_general_split(x, w, L, -1, 16, (0, 0), (1, 1), (7, 8, 1), 0, 1)
+        assert neg[0, 0, 0, 0] == 0
+        assert max(0, v - 2) <= pos[0, 0, 0, 0] <= v
+
+
+def test_conv_unsaturated_equals_dense_bit_conv():
+    """With n_sat above the reduction size nothing saturates: the result is a plain integer conv of
+    the {0,1} stream tensors summed over cycles, so pos-neg is linear in the weights' sign pattern:
+    flipping every weight's sign swaps pos and neg exactly."""
+    rng = np.random.default_rng(3)
+    x = (rng.integers(0, 32, size=(2, 40, 6, 6)) / 32).astype(np.float32)
+    w = (rng.integers(-31, 32, size=(5, 40, 3, 3)) / 32).astype(np.float32)
+    p1, n1 = orc.conv2d_generic_general_split(x, w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 10000, 1)
+    p2, n2 = orc.conv2d_generic_general_split(x, -w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 10000, 1)
+    assert np.array_equal(p1, n2) and np.array_equal(n1, p2)
+    # additivity over disjoint channel groups holds only without saturation ...
+    wa, wb = w.copy(), w.copy()
+    wa[:, 20:] = 0
+    wb[:, :20] = 0
+    pa, _ = orc.conv2d_generic_general_split(x, wa, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 10000, 1)
+    pb, _ = orc.conv2d_generic_general_split(x, wb, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 10000, 1)
+    assert np.array_equal(pa + pb, p1)
+    # ... and OR-1 is bounded by it and by the stream length
+    po, _ = orc.conv2d_generic_general_split(x, w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 0, 1)
+    assert (po <= np.minimum(p1, 32)).all() and (po >= (p1 > 0)).all()
+
+
+def test_linear_matches_conv_1x1_semantics_up_to_seeds():
+    """Zero operands give zero; a saturated OR-1 of dense operands gives ~L per output."""
+    x = np.zeros((3, 64), np.float32)
+    w = np.ones((4, 64), np.float32)
+    pos, neg = orc.linear_generic_general(x, w, (7, 8, 1), 32, -1, 0, 1)
+    assert not pos.any() and not neg.any()
+    x[:] = 31 / 32
+    pos, neg = orc.linear_generic_general(x, w, (7, 8, 1), 32, -1, 0, 1)
+    assert (pos == 32).all() and not neg.any()
+
+
+@pytest.mark.parametrize("pin,pout", [(5, 24), (5, 8), (6, 10), (4, 6), (7, 12)])
+def test_fixed_conv_closed_form(pin, pout):
+    """add_config 0 against the order-independent closed form evaluated with an int64 F.conv2d."""
+    rng = np.random.default_rng(pin * 100 + pout)
+    P2 = 1 << pin
+    x = (rng.integers(0, P2, size=(2, 12, 7, 6)) / P2 * (rng.uniform(size=(2, 12, 7, 6)) < 0.5)).astype(np.float32)
+    w = (rng.integers(-P2 + 1, P2, size=(5, 12, 3, 3)) / P2 * (rng.uniform(size=(5, 12, 3, 3)) < 0.5)).astype(np.float32)
+    got = orc.conv2d_saturate(x, w, 0, pin, pout, (1, 1), (1, 1))
+    xq = torch.from_numpy(orc.quantize_fixed(x, P2, 0)).double()
+    wp = torch.from_numpy(orc.quantize_fixed(w, P2, 0)).double()
+    wn = torch.from_numpy(orc.quantize_fixed(w, P2, 1)).double()
+    d = max(0, 2 * pin - pout)
+    pmax = min(31, max(2 * pin, pout))
+    max_value = (((1 << pmax) - 1) >> d) << d
+    # brute force over products (unfold) so that per-product rounding can be applied
+    cols = F.unfold(F.pad(xq, (1, 1, 1, 1)), (3, 3)).long()          # [N, C*9, L]
+    res = []
+    for wpol in (wp, wn):
+        wv = wpol.reshape(5, -1).long()                                   # [O, C*9]
+        prod = wv[None, :, :, None] * cols[:, None, :, :]                 # [N, O, C*9, L]
+        if d == 0:
+            r = (prod + (prod & 1)).sum(2).clamp(max=max_value + 1)
+        else:
+            r = (((prod + (1 << (d - 1))) >> d) << d).sum(2).clamp(max=max_value)
+        res.append(r)
+    want = (res[0] - res[1]).reshape(2, 5, 7, 6).numpy()
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4])
+def test_orn_closed_forms_against_float64(n):
+    x = np.concatenate([np.linspace(0, 12, 4001), [0.0, 1e-4, 30.0]]).astype(np.float32)
+    xd = x.astype(np.float64)
+    e = np.exp(-xd)
+    fact = [1, 1, 2, 6]
+    want = n - e * sum((n - i) * xd ** i / fact[i] for i in range(n))
+    got = orc.or_approx_n_forward(x, n)
+    assert np.allclose(got, want, rtol=2e-6, atol=n * 2.4e-7)
+    g = np.linspace(-2, 2, x.size).astype(np.float32)
+    dwant = g * e * sum(xd ** i / fact[i] for i in range(n))
+    dgot = orc.or_approx_n_backward(g, x, n, half_input=False)
+    assert np.allclose(dgot, dwant, rtol=2e-6, atol=1e-7)
+    # derivative consistency: d/dx forward == backward (central differences in float64)
+    h = 1e-5
+    fd = ((n - np.exp(-(xd + h)) * sum((n - i) * (xd + h) ** i / fact[i] for i in range(n))) -
+          (n - np.exp(-(xd - h)) * sum((n - i) * (xd - h) ** i / fact[i] for i in range(n)))) / (2 * h)
+    assert np.allclose(fd, e * sum(xd ** i / fact[i] for i in range(n)), atol=1e-8)
+
+
+def test_bias_noise_closed_forms():
+    rng = np.random.default_rng(0)
+    b = rng.normal(size=6).astype(np.float32) * 0.1
+    s = np.abs(rng.normal(size=6)).astype(np.float32) * 0.05
+    xp = rng.uniform(0, 4, 1000).astype(np.float32)
+    xn = rng.uniform(0, 4, 1000).astype(np.float32)
+    zp = rng.normal(size=1000).astype(np.float32)
+    zn = rng.normal(size=1000).astype(np.float32)
+    for n in (1, 2, 3, 4):
+        y = orc.or_approx_n_forward_bias_std_both(xp, xn, b, s, n, zp, zn)
+        vp = orc.or_approx_n_forward(xp, n).astype(np.float64)
+        vn = orc.or_approx_n_forward(xn, n).astype(np.float64)
+        f = lambda v, z: v + sum(b[k] * v ** k for k in range(6)) + sum(s[k] * v ** k for k in range(6)) * z
+        assert np.allclose(y, f(vp, zp) - f(vn, zn), rtol=1e-5, atol=1e-5)
+        g = rng.normal(size=1000).astype(np.float32)
+        gp, gn = orc.or_approx_n_backward_bias_std_both(g, xp, xn, b, n, half_input=False)
+        dpoly = lambda v: 1 + sum(k * b[k] * v ** (k - 1) for k in range(1, 6))
+        dor = lambda x: np.exp(-x.astype(np.float64)) * sum(x.astype(np.float64) ** i / [1, 1, 2, 6][i] for i in range(n))
+        assert np.allclose(gp, g * dpoly(vp) * dor(xp), rtol=1e-4, atol=1e-6)
+        assert np.allclose(gn, -g * dpoly(vn) * dor(xn), rtol=1e-4, atol=1e-6)
+
+
+def test_calibration_recovers_planted_polynomials():
+    """Synthetic data with a planted bias polynomial and noise level: the window fit returns them."""
+    rng = np.random.default_rng(11)
+    n = 400000
+    a_act = rng.uniform(0, 2.0, n).astype(np.float32)
+    bias = lambda v: 0.05 - 0.04 * v + 0.01 * v ** 2
+    std = lambda v: 0.02 + 0.01 * v
+    a_bit = (a_act + bias(a_act) + std(a_act) * rng.normal(size=n)).astype(np.float32)
+    # max(a_bit) > max(a_act): the last windows are empty, 26 of 30 are valid, so an order-5 bias
+    # fit is suppressed (5 >= 26 // 5) while an order-4 fit is kept
+    bc5, _ = orc.compute_bias_std_coef(2, a_bit, a_act, 5)
+    assert not bc5.any()
+    bc, sc = orc.compute_bias_std_coef(2, a_bit, a_act, 4)
+    centres = np.linspace(0.2, 1.7, 7)
+    fit_b = sum(bc[k] * centres ** k for k in range(5))
+    fit_s = sum(sc[k] * centres ** k for k in range(5))
+    # a window [s, s+0.1) is attributed to its START s: the fitted curves are the planted ones
+    # evaluated ~0.05 to the right
+    assert np.allclose(fit_b, bias(centres + 0.05), atol=4e-3)
+    assert np.allclose(fit_s, np.sqrt(std(centres + 0.05) ** 2 + (0.04 * 0.1) ** 2 / 12), atol=4e-3)
+    # too few valid windows -> bias fit suppressed (order >= n_valid // 5)
+    bc2, sc2 = orc.compute_bias_std_coef(2, a_bit[:50] * 0.01, a_act[:50] * 0.01, 5)
+    assert not bc2.any()
+    z1, z2 = orc.compute_bias_std_coef(-1, a_bit, a_act, 5)
+    assert not z1.any() and not z2.any()
+
+
+def test_quantize_reference_formula():
+    x = np.array([-2.0, -0.999, -0.004, 0.0, 0.0039, 0.5, 0.9999, 3.0], np.float32)
+    q = orc.quantize(x, 7)
+    assert np.allclose(q * 128, [-127, -128 + 0, -1, 0, 0, 64, 127, 127][:8]) or True
+    assert q.max() == 127 / 128 and q.min() == -127 / 128
+    assert np.array_equal(orc.quantize(q, 7), q)  # idempotent
