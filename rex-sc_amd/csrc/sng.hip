@@ -6,6 +6,8 @@
 //
 // Semantics follow the reference CPU extension: sc_conv.cpp:42-200 (conv), sc_matmul.cpp:3-383
 // (linear); quantisation sc_conv.cpp:316-320.
+#include <utility>
+
 #include "sng.h"
 #include "profile.h"
 
@@ -73,6 +75,60 @@ __device__ __forceinline__ void load_tables_to_lds(const SeqTable *tab, uint8_t 
     for (int i = threadIdx.x; i < 64; i += blockDim.x) dsti[i] = srci[i];
 }
 
+
+// One 64-channel group, up to 32 consecutive slots [s0, s0+ns): lane = channel holds its quantised
+// value v and its LFSR cycle position pos.  Each slot is one v_cmp whose 64-bit lane mask is the
+// pair of stream words; the masks are deposited with v_writelane so that afterwards LANE s holds
+// the two words of SLOT s0+s (lo = channels 0..31, hi = channels 32..63).
+//
+// v_writelane_b32 with an immediate lane select puts a wave-uniform value into lane LANE of a VGPR.
+// Only one SGPR may feed a VALU instruction on this hardware, so the lane select cannot be a second
+// SGPR.  The mask comes straight from a v_cmp: a VALU write of an SGPR needs two wait states before
+// another VALU instruction reads it, and the compiler does not track hazards into inline asm, hence
+// the s_nop.
+template <int LANE>
+__device__ __forceinline__ void write_lanes(uint32_t &lo, uint32_t &hi, unsigned long long mask)
+{
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass of hipcc parses device functions too
+    asm("s_nop 1\n\tv_writelane_b32 %0, %2, %4\n\tv_writelane_b32 %1, %3, %4"
+        : "+v"(lo), "+v"(hi)
+        : "s"((uint32_t)mask), "s"((uint32_t)(mask >> 32)), "n"(LANE));
+#endif
+}
+
+template <int S>
+__device__ __forceinline__ void gen_slot_fast(const uint8_t *p, int v, uint32_t &lo, uint32_t &hi)
+{
+    write_lanes<S>(lo, hi, __ballot(v > (int)p[S]));
+}
+
+template <int... S>
+__device__ __forceinline__ void gen_slots_fast(const uint8_t *p, int v, uint32_t &lo, uint32_t &hi,
+                                               std::integer_sequence<int, S...>)
+{
+    (gen_slot_fast<S>(p, v, lo, hi), ...);
+}
+
+__device__ __forceinline__ void gen_slots32(const uint8_t *s_seq, int pos, int v, const GenParams &gp, int s0, int ns,
+                                            uint32_t &lo, uint32_t &hi)
+{
+    lo = 0; hi = 0;
+    const bool ident = gp.slot_div == 1 && gp.slot_mul == 1 && gp.slot_mod == 1; // slot == cycle
+    if (ident && !gp.prog && ns == 32) {
+        gen_slots_fast(s_seq + pos + s0, v, lo, hi, std::make_integer_sequence<int, 32>{});
+    } else {
+        const int lane = threadIdx.x & 63;
+        for (int s = 0; s < ns; s++) {
+            const int t = slot_cycle(gp, s0 + s);
+            const int st = s_seq[pos + t];
+            int vv = v;
+            if (gp.prog) { const int sh = prog_shift(gp, t); vv = (v >> sh) << sh; }
+            const unsigned long long m = __ballot(vv > st);
+            if (lane == s) { lo = (uint32_t)m; hi = (uint32_t)(m >> 32); }
+        }
+    }
+}
+
 // ---- activation SNG --------------------------------------------------------------------------
 // Block: 256 threads.  Tile: 64 consecutive positions pp of the PADDED plane of image n,
 // one channel chunk zg (32*ZC channels).
@@ -80,6 +136,9 @@ __device__ __forceinline__ void load_tables_to_lds(const SeqTable *tab, uint8_t 
 constexpr int ACT_TILE = 64;
 constexpr int ACT_SLOT_GROUP = 32;
 constexpr int QPITCH = ACT_TILE + 4; // bytes per channel row in LDS; 17 dwords -> conflict-free column reads
+// dwords between the rows of two slots in the LDS staging buffer: +2 spreads the per-lane (= per-slot)
+// 8-byte writes over the banks
+template <int ZC> constexpr int act_pitch() { return ACT_TILE * ZC + 2; }
 
 template <int ZC>
 __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ x, uint32_t *__restrict__ A,
@@ -90,7 +149,8 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
     __shared__ __attribute__((aligned(16))) uint8_t s_seq[SEQ_LEN];
     __shared__ __attribute__((aligned(16))) uint8_t s_inv[256];
     __shared__ __attribute__((aligned(16))) uint8_t s_q[CCH * QPITCH];
-    __shared__ __attribute__((aligned(16))) uint32_t s_stage[ACT_SLOT_GROUP * ACT_TILE * ZC];
+    constexpr int PITCH = act_pitch<ZC>();
+    __shared__ __attribute__((aligned(16))) uint32_t s_stage[ACT_SLOT_GROUP * PITCH];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int pp0 = blockIdx.x * ACT_TILE;
@@ -153,17 +213,12 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
                 int sd = cmod[h] + pmod;
                 if (sd >= gp.seed_mod) sd -= gp.seed_mod;
                 const int pos = s_inv[sd + 1] + 1; // state of cycle t is seq[pos + t]
-                for (int s = 0; s < ns; s++) {
-                    const int t = slot_cycle(gp, s0 + s);
-                    const int st = s_seq[pos + t];
-                    int vv = v;
-                    if (gp.prog) { const int sh = prog_shift(gp, t); vv = (v >> sh) << sh; }
-                    const unsigned long long m = __ballot(vv > st);
-                    if (lane == 0) {
-                        uint32_t *dst = &s_stage[(s * ACT_TILE + j) * ZC + h * 2];
-                        dst[0] = (uint32_t)m;
-                        if (ZC > 1) dst[1] = (uint32_t)(m >> 32);
-                    }
+                uint32_t lo, hi;
+                gen_slots32(s_seq, pos, v, gp, s0, ns, lo, hi);
+                if (lane < ns) {
+                    uint32_t *dst = &s_stage[lane * PITCH + j * ZC + h * 2];
+                    dst[0] = lo;
+                    if (ZC > 1) dst[1] = hi;
                 }
             }
         }
@@ -172,7 +227,7 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
         const int run = npix * ZC;
         for (int s = 0; s < ns; s++) {
             uint32_t *dst = A + (long)(s0 + s) * geo.slot_stride + (((long)n * geo.ZG + zg) * HpWp + pp0) * ZC;
-            for (int i = tid; i < run; i += 256) dst[i] = s_stage[s * ACT_TILE * ZC + i];
+            for (int i = tid; i < run; i += 256) dst[i] = s_stage[s * PITCH + i];
         }
         __syncthreads();
     }
@@ -200,6 +255,7 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
     const int og = blockIdx.x, ky = blockIdx.y, zg = blockIdx.z;
     const int KW = geo.KW;
     const int row = W_OG * 2 * KW * ZC; // words per slot handled by this block
+    const int pitch = row + 2;          // LDS row pitch (bank spreading for the per-slot writes)
     const float S = (float)gp.scale;
 
     load_tables_to_lds(tables + seq_index(gp.lb, gp.acc), s_seq, s_inv);
@@ -226,25 +282,20 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
             // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
             const int sd = (int)((13L + (long)c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
             const int pos = s_inv[sd + 1] + 1;
-            for (int s = 0; s < ns; s++) {
-                const int t = slot_cycle(gp, s0 + s);
-                const int st = s_seq[pos + t];
-                int ap = vp, an = vn;
-                if (gp.prog) { const int sh = prog_shift(gp, t); ap = (vp >> sh) << sh; an = (vn >> sh) << sh; }
-                const unsigned long long mp = __ballot(ap > st);
-                const unsigned long long mn = __ballot(an > st);
-                if (lane == 0) {
-                    uint32_t *dp = &s_stage[s * row + ((ol * 2 + 0) * KW + kx) * ZC + h * 2];
-                    uint32_t *dn = &s_stage[s * row + ((ol * 2 + 1) * KW + kx) * ZC + h * 2];
-                    dp[0] = (uint32_t)mp; dn[0] = (uint32_t)mn;
-                    if (ZC > 1) { dp[1] = (uint32_t)(mp >> 32); dn[1] = (uint32_t)(mn >> 32); }
-                }
+            uint32_t plo, phi, nlo, nhi;
+            gen_slots32(s_seq, pos, vp, gp, s0, ns, plo, phi);
+            gen_slots32(s_seq, pos, vn, gp, s0, ns, nlo, nhi);
+            if (lane < ns) {
+                uint32_t *dp = &s_stage[lane * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2];
+                uint32_t *dn = &s_stage[lane * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2];
+                dp[0] = plo; dn[0] = nlo;
+                if (ZC > 1) { dp[1] = phi; dn[1] = nhi; }
             }
         }
         __syncthreads();
         for (int s = 0; s < ns; s++) {
             uint32_t *dst = Wst + ((((long)(s0 + s) * geo.KH + ky) * geo.ZG + zg) * geo.O_pad + og * W_OG) * 2 * KW * ZC;
-            for (int i = tid; i < row; i += 256) dst[i] = s_stage[s * row + i];
+            for (int i = tid; i < row; i += 256) dst[i] = s_stage[s * pitch + i];
         }
         __syncthreads();
     }
@@ -283,7 +334,7 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
                          const GenParams &gp, hipStream_t stream)
 {
     dim3 grid(geo.O_pad / W_OG, geo.KH, geo.ZG);
-    const size_t row_bytes = sizeof(uint32_t) * W_OG * 2 * geo.KW * ZC;
+    const size_t row_bytes = sizeof(uint32_t) * (W_OG * 2 * geo.KW * ZC + 2);
     int slot_group = (int)((60 * 1024 - SEQ_LEN - 256) / row_bytes);
     if (slot_group > W_SLOT_GROUP) slot_group = W_SLOT_GROUP;
     REXSC_CHECK_ARG(slot_group >= 1, "weight SNG: kernel width %d too large for LDS staging", geo.KW);
