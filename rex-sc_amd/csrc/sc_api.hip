@@ -24,7 +24,7 @@ constexpr size_t WS_ALIGN = 256;
 // Activation streams of one batch chunk are kept below this many bytes; larger batches are
 // processed chunk by chunk with the weight streams generated once.
 constexpr size_t ACT_STREAM_CAP = (size_t)1 << 30;
-constexpr int TARGET_WAVES = 4096; // ~4 waves per SIMD on 256 CUs
+constexpr int TARGET_WAVES = 3072; // 3 resident waves per SIMD on 256 CUs x 4 SIMDs
 
 struct ScPlan {
     // generators
@@ -147,15 +147,21 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     cp.mode = (linear && bin_config < 0) ? 1 : 0;
     cp.out_channels_last = linear ? 1 : act_cl; // linear output is [B][O]
 
-    // tiling: pixels per lane and slot splits
+    // tiling.  A block is NS waves sharing one tile of 64*px pixels x OT channels, each wave taking
+    // 1/NS of the stream slots (partials meet in LDS).  Two pixels per lane halve the scalar weight
+    // traffic per VALU instruction.  The launch should be several rounds of the ~3072 resident waves
+    // (256 CUs x 4 SIMDs x 3) so that its tail is short; what the tiles and NS do not supply comes
+    // from splitting the slots over blocks as well (partials merged by the finalize kernel).
     const int o_tiles = O_pad / OT;
-    long waves1 = (long)ceil_div(cp.M, 256) * 4 * o_tiles;
-    cp.px = (!pl.wide && waves1 >= 2L * TARGET_WAVES) ? 2 : 1;
-    long waves = (long)ceil_div(cp.M, 256 * cp.px) * 4 * o_tiles;
+    cp.px = (!pl.wide && cp.M >= 1024) ? 2 : 1;
+    cp.ns = n_slots >= 8 ? 4 : (n_slots >= 2 ? 2 : 1);
+    long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
     int splits = 1;
-    if (pl.tuned && waves < TARGET_WAVES / 2) {
-        splits = (int)((TARGET_WAVES / 2 + waves - 1) / waves);
-        if (splits > n_slots) splits = n_slots;
+    const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
+    if (pl.tuned && waves < 4L * TARGET_WAVES) {
+        splits = (int)((4L * TARGET_WAVES + waves - 1) / waves);
+        if (splits > max_splits) splits = max_splits;
+        if (splits > 8) splits = 8;
     }
     cp.slots_per_split = ceil_div(n_slots, splits);
     cp.splits = ceil_div(n_slots, cp.slots_per_split);
@@ -163,7 +169,8 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     if (!pl.tuned) { cp.direct = 1; cp.splits = 1; cp.slots_per_split = n_slots; }
 
     // workspace
-    const size_t w_bytes = (size_t)n_slots * KH * ZG * O_pad * 2 * KW * ZC * 4;
+    // + one chunk: the compute kernel's weight prefetch reads one batch past the last chunk
+    const size_t w_bytes = ((size_t)n_slots * KH * ZG + 1) * O_pad * 2 * KW * ZC * 4;
     const size_t a_bytes = (size_t)n_slots * ag.slot_stride * 4;
     const size_t part_bytes = cp.direct ? 0 : (size_t)(pl.wide ? 2 : 1) * cp.splits * O_pad * cp.M * 4;
     pl.off_w = 0;

@@ -20,6 +20,7 @@ struct ComputeParams {
     int direct;       // 1: the compute kernel writes the int16 outputs itself
     int out_channels_last;
     int px;           // pixels per lane (1 or 2)
+    int ns;           // waves per block; they split the slots of the block among themselves
     int m_tiles, o_tiles; // filled by the launcher
 };
 

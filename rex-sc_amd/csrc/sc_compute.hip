@@ -11,8 +11,13 @@
 //                     16-bit wrap-around of the running sum.
 //   reduction order = slot (outer) -> kernel row ky -> channel chunk zg (runtime loops);
 //                     inside a chunk everything is unrolled: OT x KW x ZC x PX (and+bcnt) x 2.
-//   grid            = pixel tiles x output-channel tiles x slot splits, remapped so that the
-//                     blocks sharing a pixel tile run on the same XCD (shared L2).
+//   block           = NS waves that share one tile of 64*PX pixels x OT channels and split the
+//                     stream slots among themselves; their partial sums meet in LDS, so the final
+//                     int16 results are written once and no partial traffic reaches HBM.  Short
+//                     waves (slots/NS each) keep the tail of the launch small: with ~1000 SIMDs
+//                     and 3 resident waves each, whole-reduction waves would quantise badly.
+//   grid            = pixel tiles x output-channel tiles x (optional) global slot splits, remapped
+//                     so that the blocks sharing a pixel tile run on the same XCD (shared L2).
 #include "sc_compute.h"
 #include "profile.h"
 
@@ -53,16 +58,61 @@ __device__ __forceinline__ void load_words(const uint32_t *__restrict__ p, uint3
     }
 }
 
-constexpr int CB = 256; // threads per block
+// Output channels per weight batch: the largest power of two whose batch (G*2*KWZ dwords) fits 32
+// SGPRs, at least 1 and at most OT/2 (so that a chunk holds an even number of batches).
+constexpr int pick_group(int kwz, int ot)
+{
+    int g = 1;
+    while (g * 2 <= ot / 2 && g * 2 * 2 * kwz <= 32) g *= 2;
+    return g;
+}
+
+// count += popcount(a & w): v_and_b32 (weight word as the scalar operand) + v_bcnt_u32_b32 with its
+// accumulate input.  The accumulate form is spelled out because the compiler otherwise reassociates
+// chains of popcounts into popcount+popcount+add3, which costs 3 instructions per 2 words.
+__device__ __forceinline__ void and_popc_acc(uint32_t &count, uint32_t a, uint32_t w)
+{
+    const uint32_t t = a & w;
+#if defined(__HIP_DEVICE_COMPILE__) // the host pass of hipcc parses device functions too
+    asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(count) : "v"(t));
+#else
+    count += __builtin_popcount(t);
+#endif
+}
+
+// One weight batch: G output channels starting at o0, both polarities, all KWZ words, PX pixels.
+// wb holds [g][pol][j].
+template <int PX, int OT, int KWZ, int G>
+__device__ __forceinline__ void compute_batch(const uint32_t (&a)[PX][KWZ], const uint32_t (&wb)[G * 2 * KWZ],
+                                              uint32_t (&cp)[PX][OT], uint32_t (&cn)[PX][OT], int o0)
+{
+#pragma unroll
+    for (int g = 0; g < G; g++)
+#pragma unroll
+        for (int j = 0; j < KWZ; j++) {
+            const uint32_t wp = wb[(g * 2 + 0) * KWZ + j];
+            const uint32_t wn = wb[(g * 2 + 1) * KWZ + j];
+#pragma unroll
+            for (int px = 0; px < PX; px++) {
+                and_popc_acc(cp[px][o0 + g], a[px][j], wp);
+                and_popc_acc(cn[px][o0 + g], a[px][j], wn);
+            }
+        }
+}
+
+constexpr int MAX_NS = 4; // waves per block (each takes a share of the stream slots)
+// s_waitcnt immediate: lgkmcnt(0), vmcnt and expcnt left at their maxima (not waited for)
+constexpr int WAIT_LGKM0 = 0xC07F;
 
 template <int KW, int ZC, int PX, int OT, bool WIDE>
-__global__ __launch_bounds__(CB) void sc_compute_kernel(const uint32_t *__restrict__ A,
+__global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t *__restrict__ A,
                                                         const uint32_t *__restrict__ Wst, ComputeParams p,
                                                         uint32_t *__restrict__ part, int16_t *__restrict__ out_pos,
                                                         int16_t *__restrict__ out_neg, int16_t *__restrict__ out_diff)
 {
     constexpr int KWZ = KW * ZC;
-    constexpr int BM = CB * PX;
+    constexpr int BM = 64 * PX;            // pixels per block (every wave of the block covers all of them)
+    __shared__ uint32_t s_red[MAX_NS][WIDE ? 2 : 1][PX * OT][64];
 
     // XCD-aware block remap: hardware deals consecutive block ids round-robin over 8 XCDs;
     // give each XCD a contiguous range of logical ids (o-tiles of one pixel tile are adjacent).
@@ -73,12 +123,15 @@ __global__ __launch_bounds__(CB) void sc_compute_kernel(const uint32_t *__restri
     const int mtile = bid % p.m_tiles;
     const int split = bid / p.m_tiles;
 
-    const int tid = threadIdx.x;
+    const int lane = threadIdx.x & 63, ns = blockDim.x >> 6;
+    // wave index, made provably wave-uniform so that everything derived from it (slot range, weight
+    // addresses) stays in SGPRs and the weight loads stay scalar
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int abase[PX]; // word offset of the lane's pixel inside one slot, for ky = 0, zg = 0
     int mpix[PX];
 #pragma unroll
     for (int px = 0; px < PX; px++) {
-        const int m = mtile * BM + px * CB + tid;
+        const int m = mtile * BM + px * 64 + lane;
         mpix[px] = m;
         const int mm = m < p.M ? m : p.M - 1;
         const int n = mm / p.HoWo, r = mm - n * p.HoWo;
@@ -93,112 +146,183 @@ __global__ __launch_bounds__(CB) void sc_compute_kernel(const uint32_t *__restri
 #pragma unroll
         for (int o = 0; o < OT; o++) { acc[px][o] = 0; if (WIDE) accw[px][o] = 0; }
 
-    const int s_begin = split * p.slots_per_split;
-    const int s_end = min(p.n_slots, s_begin + p.slots_per_split);
+    // slots of this block, then of this wave
+    const int sb_begin = split * p.slots_per_split;
+    const int sb_end = min(p.n_slots, sb_begin + p.slots_per_split);
+    const int per_wave = (sb_end - sb_begin + ns - 1) / ns;
+    const int s_begin = min(sb_end, sb_begin + wave * per_wave);
+    const int s_end = min(sb_end, s_begin + per_wave);
     const int chunk_stride = p.Hp * p.Wp * ZC; // words between zg planes
+    const int row_stride = p.Wp * ZC;          // words between kernel rows
     const long w_chunk_words = (long)p.O_pad * 2 * KWZ;
 
-    for (int slot = s_begin; slot < s_end; slot++) {
-        uint32_t cp[PX][OT], cn[PX][OT];
+    // The reduction is walked chunk by chunk: chunk q = (slot, ky, zg) in that order, which is also
+    // the order of the weight stream in memory.  Two software pipelines hide latency:
+    //  * activations: the words of chunk q+1 are loaded into a second register set while chunk q
+    //    is being computed;
+    //  * weights: each chunk is consumed in batches of G output channels (BW dwords); the scalar
+    //    loads of batch b+1 are issued before the VALU work of batch b.  Scalar loads return out of
+    //    order, so a wave can only wait for all of them: issuing exactly one batch ahead keeps the
+    //    wait at the top of every batch short.  The last batch of a chunk prefetches the first
+    //    batch of the next chunk (the weight buffer is padded by one chunk for the final over-read).
+    constexpr int G = pick_group(KWZ, OT);
+    constexpr int BW = G * 2 * KWZ;  // dwords per weight batch
+    constexpr int NB = OT / G;       // batches per chunk (even)
+    static_assert(NB % 2 == 0, "the batch ping-pong needs an even number of batches per chunk");
+
+    const int chunks_per_slot = p.KH * p.ZG;
+    const int q_begin = s_begin * chunks_per_slot, q_end = s_end * chunks_per_slot;
+    const uint32_t *w_q = Wst + (long)q_begin * w_chunk_words + (long)otile * OT * 2 * KWZ;
+
+    uint32_t cp[PX][OT], cn[PX][OT];
+#pragma unroll
+    for (int px = 0; px < PX; px++)
+#pragma unroll
+        for (int o = 0; o < OT; o++) { cp[px][o] = 0; cn[px][o] = 0; }
+
+    uint32_t a_cur[PX][KWZ], a_nxt[PX][KWZ];
+    uint32_t wb0[BW], wb1[BW];
+    int slot = s_begin, ky = 0, zg = 0;
+    if (s_begin < s_end) { // wave-uniform
+        const uint32_t *a_chunk = A + (long)slot * p.a_slot_stride;
 #pragma unroll
         for (int px = 0; px < PX; px++)
 #pragma unroll
-            for (int o = 0; o < OT; o++) { cp[px][o] = 0; cn[px][o] = 0; }
+            for (int kx = 0; kx < KW; kx++) load_words<ZC>(a_chunk + abase[px] + kx * ZC, &a_cur[px][kx * ZC]);
+#pragma unroll
+        for (int e = 0; e < BW; e++) wb0[e] = w_q[e];
+    }
 
-        const uint32_t *a_slot = A + (long)slot * p.a_slot_stride;
-        const uint32_t *w_slot = Wst + (long)slot * p.KH * p.ZG * w_chunk_words + (long)otile * OT * 2 * KWZ;
-        for (int ky = 0; ky < p.KH; ky++) {
-            for (int zg = 0; zg < p.ZG; zg++) {
-                uint32_t a[PX][KWZ];
-#pragma unroll
-                for (int px = 0; px < PX; px++) {
-                    const uint32_t *ap = a_slot + abase[px] + zg * chunk_stride + ky * p.Wp * ZC;
-#pragma unroll
-                    for (int kx = 0; kx < KW; kx++) load_words<ZC>(ap + kx * ZC, &a[px][kx * ZC]);
-                }
-                const uint32_t *wc = w_slot + (long)(ky * p.ZG + zg) * w_chunk_words;
-#pragma unroll
-                for (int o = 0; o < OT; o++) {
-#pragma unroll
-                    for (int j = 0; j < KWZ; j++) {
-                        const uint32_t wp = wc[(o * 2 + 0) * KWZ + j];
-                        const uint32_t wn = wc[(o * 2 + 1) * KWZ + j];
-#pragma unroll
-                        for (int px = 0; px < PX; px++) {
-                            cp[px][o] += __builtin_popcount(a[px][j] & wp);
-                            cn[px][o] += __builtin_popcount(a[px][j] & wn);
-                        }
-                    }
-                }
-            }
-        }
-        // per-slot saturation and accumulation
-        if (!WIDE) {
-            if (p.mode == 0) {
-#pragma unroll
-                for (int px = 0; px < PX; px++)
-#pragma unroll
-                    for (int o = 0; o < OT; o++) {
-                        const uint32_t c = cp[px][o] | (cn[px][o] << 16);
-                        acc[px][o] = pk_add_u16(acc[px][o], pk_min_u16(c, p.nn));
-                    }
-            } else { // [count >= n] = min(count, n) - min(count, n-1)
-#pragma unroll
-                for (int px = 0; px < PX; px++)
-#pragma unroll
-                    for (int o = 0; o < OT; o++) {
-                        const uint32_t c = cp[px][o] | (cn[px][o] << 16);
-                        const uint32_t d = pk_sub_u16(pk_min_u16(c, p.nn), pk_min_u16(c, p.nn - 0x00010001u));
-                        acc[px][o] = pk_add_u16(acc[px][o], d);
-                    }
-            }
-        } else {
-            const uint32_t n = p.nn & 0xffffu;
+    for (int q = q_begin; q < q_end; q++) {
+        // coordinates of the next chunk
+        int zg_n = zg + 1, ky_n = ky, slot_n = slot;
+        if (zg_n == p.ZG) { zg_n = 0; ky_n++; if (ky_n == p.KH) { ky_n = 0; slot_n++; } }
+        const bool slot_done = (zg_n == 0 && ky_n == 0);
+        {
+            // prefetch its activation words (the last chunk re-reads itself: harmless)
+            const bool has_next = q + 1 < q_end;
+            const int sl = has_next ? slot_n : slot, kk = has_next ? ky_n : ky, zz = has_next ? zg_n : zg;
+            const uint32_t *a_chunk = A + (long)sl * p.a_slot_stride + zz * chunk_stride + kk * row_stride;
 #pragma unroll
             for (int px = 0; px < PX; px++)
 #pragma unroll
-                for (int o = 0; o < OT; o++) {
-                    if (p.mode == 0) {
-                        acc[px][o] += min(cp[px][o], n);
-                        accw[px][o] += min(cn[px][o], n);
-                    } else {
-                        acc[px][o] += cp[px][o] >= n;
-                        accw[px][o] += cn[px][o] >= n;
-                    }
-                }
+                for (int kx = 0; kx < KW; kx++) load_words<ZC>(a_chunk + abase[px] + kx * ZC, &a_nxt[px][kx * ZC]);
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < NB; b += 2) {
+            // batch b lives in wb0, batch b+1 in wb1
+            // Make sure the batch about to be used has landed BEFORE the next one is requested: the
+            // compiler would otherwise place this wait after the request and wait for both.
+            __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
+            {
+                const uint32_t *src = w_q + (b + 1) * BW;
+#pragma unroll
+                for (int e = 0; e < BW; e++) wb1[e] = src[e];
+            }
+            __builtin_amdgcn_sched_barrier(0); // keep the prefetch above the VALU work it overlaps with
+            compute_batch<PX, OT, KWZ, G>(a_cur, wb0, cp, cn, b * G);
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
+            {
+                const uint32_t *src = (b + 2 < NB) ? w_q + (b + 2) * BW : w_q + w_chunk_words;
+#pragma unroll
+                for (int e = 0; e < BW; e++) wb0[e] = src[e];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            compute_batch<PX, OT, KWZ, G>(a_cur, wb1, cp, cn, (b + 1) * G);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (slot_done) {
+            // per-slot saturation and accumulation
+            if (!WIDE) {
+                if (p.mode == 0) {
+#pragma unroll
+                    for (int px = 0; px < PX; px++)
+#pragma unroll
+                        for (int o = 0; o < OT; o++) {
+                            const uint32_t c = cp[px][o] | (cn[px][o] << 16);
+                            acc[px][o] = pk_add_u16(acc[px][o], pk_min_u16(c, p.nn));
+                        }
+                } else { // [count >= n] = min(count, n) - min(count, n-1)
+#pragma unroll
+                    for (int px = 0; px < PX; px++)
+#pragma unroll
+                        for (int o = 0; o < OT; o++) {
+                            const uint32_t c = cp[px][o] | (cn[px][o] << 16);
+                            const uint32_t d = pk_sub_u16(pk_min_u16(c, p.nn), pk_min_u16(c, p.nn - 0x00010001u));
+                            acc[px][o] = pk_add_u16(acc[px][o], d);
+                        }
+                }
+            } else {
+                const uint32_t n = p.nn & 0xffffu;
+#pragma unroll
+                for (int px = 0; px < PX; px++)
+#pragma unroll
+                    for (int o = 0; o < OT; o++) {
+                        if (p.mode == 0) {
+                            acc[px][o] += min(cp[px][o], n);
+                            accw[px][o] += min(cn[px][o], n);
+                        } else {
+                            acc[px][o] += cp[px][o] >= n;
+                            accw[px][o] += cn[px][o] >= n;
+                        }
+                    }
+            }
+#pragma unroll
+            for (int px = 0; px < PX; px++)
+#pragma unroll
+                for (int o = 0; o < OT; o++) { cp[px][o] = 0; cn[px][o] = 0; }
+        }
+#pragma unroll
+        for (int px = 0; px < PX; px++)
+#pragma unroll
+            for (int j = 0; j < KWZ; j++) a_cur[px][j] = a_nxt[px][j];
+        w_q += w_chunk_words;
+        slot = slot_n; ky = ky_n; zg = zg_n;
     }
 
-    // epilogue
-    if (p.direct) {
+    // epilogue: sum the NS partial tiles in LDS; each wave then finishes every ns-th accumulator
+    if (ns > 1) {
 #pragma unroll
-        for (int px = 0; px < PX; px++) {
-            const int m = mpix[px];
-            if (m >= p.M) continue;
-            const int n = m / p.HoWo, r = m - n * p.HoWo;
+        for (int px = 0; px < PX; px++)
 #pragma unroll
             for (int o = 0; o < OT; o++) {
-                const int oo = otile * OT + o;
+                s_red[wave][0][px * OT + o][lane] = acc[px][o];
+                if (WIDE) s_red[wave][1][px * OT + o][lane] = accw[px][o];
+            }
+        __syncthreads();
+    }
+    const long plane = (long)p.splits * p.O_pad * p.M;
+#pragma unroll
+    for (int px = 0; px < PX; px++) {
+        const int m = mpix[px];
+        const int n = m / p.HoWo, r = m - n * p.HoWo;
+#pragma unroll
+        for (int o = 0; o < OT; o++) {
+            if (((px * OT + o) % ns) != wave) continue; // wave-uniform
+            uint32_t v = acc[px][o], vw = WIDE ? accw[px][o] : 0;
+            if (ns > 1) {
+                v = 0; vw = 0;
+                for (int w = 0; w < ns; w++) {
+                    if (WIDE) { v += s_red[w][0][px * OT + o][lane]; vw += s_red[w][1][px * OT + o][lane]; }
+                    else v = pk_add_u16(v, s_red[w][0][px * OT + o][lane]);
+                }
+            }
+            if (m >= p.M) continue;
+            const int oo = otile * OT + o;
+            if (p.direct) {
                 if (oo >= p.O) continue;
                 const long idx = p.out_channels_last ? (long)m * p.O + oo : ((long)n * p.O + oo) * p.HoWo + r;
-                const int16_t vp = (int16_t)(acc[px][o] & 0xffffu), vn = (int16_t)(acc[px][o] >> 16);
+                const int16_t vp = (int16_t)(v & 0xffffu), vn = (int16_t)(v >> 16);
                 if (out_pos) out_pos[idx] = vp;
                 if (out_neg) out_neg[idx] = vn;
                 if (out_diff) out_diff[idx] = (int16_t)(vp - vn);
-            }
-        }
-    } else {
-        // partial sums: part[plane][split][o][m]; plane 1 only in WIDE mode
-        const long plane = (long)p.splits * p.O_pad * p.M;
-#pragma unroll
-        for (int px = 0; px < PX; px++) {
-            const int m = mpix[px];
-            if (m >= p.M) continue;
-#pragma unroll
-            for (int o = 0; o < OT; o++) {
-                const long idx = ((long)split * p.O_pad + otile * OT + o) * p.M + m;
-                part[idx] = acc[px][o];
-                if (WIDE) part[plane + idx] = accw[px][o];
+            } else {
+                // partial sums of a global slot split: part[plane][split][o][m]; plane 1 only in WIDE mode
+                const long idx = ((long)split * p.O_pad + oo) * p.M + m;
+                part[idx] = v;
+                if (WIDE) part[plane + idx] = vw;
             }
         }
     }
@@ -274,8 +398,9 @@ template <int KW, int ZC, int PX, int OT, bool WIDE>
 static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams p, uint32_t *part, int16_t *out_pos,
                           int16_t *out_neg, int16_t *out_diff, hipStream_t stream)
 {
-    p.m_tiles = ceil_div(p.M, CB * PX);
+    p.m_tiles = ceil_div(p.M, 64 * PX);
     p.o_tiles = p.O_pad / OT;
+    REXSC_CHECK_ARG(p.ns >= 1 && p.ns <= MAX_NS, "SC compute: %d waves per block not supported", p.ns);
     const long blocks = (long)p.m_tiles * p.o_tiles * p.splits;
     REXSC_CHECK_ARG(blocks < (1L << 30), "SC compute: grid too large (%ld blocks)", blocks);
     const int grid = (int)align_up((size_t)blocks, 8);
@@ -283,7 +408,7 @@ static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams 
     if (!name[0]) snprintf(name, sizeof(name), "sc_compute<%d,%d,%d,%d,%d>", KW, ZC, PX, OT, (int)WIDE);
     // algorithmic lane-ops: (and + popcount-accumulate) x 2 polarities per 32-channel word
     ProfScope prof(name, 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
-    hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, WIDE>), dim3(grid), dim3(CB), 0, stream, A, Wst, p, part,
+    hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, WIDE>), dim3(grid), dim3(64 * p.ns), 0, stream, A, Wst, p, part,
                        out_pos, out_neg, out_diff);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
