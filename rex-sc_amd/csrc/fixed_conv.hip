@@ -141,6 +141,175 @@ __global__ __launch_bounds__(256) void fixed_conv_kernel(const int32_t *__restri
     }
 }
 
+
+// ---- int8 MFMA path for the closed form ----------------------------------------------------------
+// Valid when add_config = 0, d = 0, operands fit int8 (precision_in <= 7) and the clamp cannot fire
+// (C*KH*KW*((2^pin-1)^2+1) < max_value+1).  Then pos - neg collapses to ONE signed contraction with
+// the reduction doubled:  out = sum a*w  +  sum (a&1) * sgn(w)*(|w|&1).
+//
+// Operands are re-laid-out once, channel-blocked by 8 so that every MFMA operand fetch is an
+// 8-byte load and adjacent lanes read adjacent memory:
+//   xq8[n][cb][yp][xp][8]   int8, zero padded plane; blocks [0,CBV) values, [CBV,2*CBV) parities
+//   wq8[cb][ky][kx][o_pad][8] int8, same block order
+// GEMM orientation: MFMA rows = output channels (weights are the A operand), MFMA columns =
+// pixels (activations are the B operand), so that the 32 lanes of a half-wave hold 32
+// consecutive pixels of one output channel and the int32 NCHW stores are 128-byte runs.
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct Fixed8Params {
+    int N, C, H, W, O, O_pad, KH, KW;
+    int pad_h, pad_w, s0, s1, Hp, Wp, Ho, Wo;
+    int CBV, CB; // value blocks, total blocks (= 2*CBV)
+    int M;       // N*Ho*Wo
+    float P2;
+};
+
+__global__ __launch_bounds__(256) void fixed_pack_act8_kernel(const float *__restrict__ x, int8_t *__restrict__ xq8,
+                                                              Fixed8Params p)
+{
+    // one thread per (n, cbv, yp, xp): 8 channels -> one value block and one parity block
+    const long total = (long)p.N * p.CBV * p.Hp * p.Wp;
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int xp = (int)(i % p.Wp);
+        const int yp = (int)((i / p.Wp) % p.Hp);
+        const int cbv = (int)((i / ((long)p.Wp * p.Hp)) % p.CBV);
+        const int n = (int)(i / ((long)p.Wp * p.Hp * p.CBV));
+        const int y = yp - p.pad_h, xx = xp - p.pad_w;
+        const bool inb = y >= 0 && y < p.H && xx >= 0 && xx < p.W;
+        uint64_t vals = 0, pars = 0;
+        if (inb) {
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int c = cbv * 8 + k;
+                if (c < p.C) {
+                    const int q = quant_round_pos(x[(((long)n * p.C + c) * p.H + y) * p.W + xx], p.P2);
+                    vals |= (uint64_t)(uint8_t)q << (8 * k);
+                    pars |= (uint64_t)(q & 1) << (8 * k);
+                }
+            }
+        }
+        const long plane = (long)p.Hp * p.Wp;
+        uint64_t *dst = reinterpret_cast<uint64_t *>(xq8);
+        dst[((long)n * p.CB + cbv) * plane + (long)yp * p.Wp + xp] = vals;
+        dst[((long)n * p.CB + p.CBV + cbv) * plane + (long)yp * p.Wp + xp] = pars;
+    }
+}
+
+__global__ __launch_bounds__(256) void fixed_pack_w8_kernel(const float *__restrict__ w, int8_t *__restrict__ wq8,
+                                                            Fixed8Params p)
+{
+    const long total = (long)p.CBV * p.KH * p.KW * p.O_pad;
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const int o = (int)(i % p.O_pad);
+        const int kx = (int)((i / p.O_pad) % p.KW);
+        const int ky = (int)((i / ((long)p.O_pad * p.KW)) % p.KH);
+        const int cbv = (int)(i / ((long)p.O_pad * p.KW * p.KH));
+        uint64_t vals = 0, pars = 0;
+        if (o < p.O) {
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const int c = cbv * 8 + k;
+                if (c < p.C) {
+                    const float f = w[(((long)o * p.C + c) * p.KH + ky) * p.KW + kx];
+                    const int q = quant_round_pos(f, p.P2) - quant_round_neg(f, p.P2); // signed
+                    const int par = (q & 1) ? (q < 0 ? -1 : 1) : 0;
+                    vals |= (uint64_t)(uint8_t)(int8_t)q << (8 * k);
+                    pars |= (uint64_t)(uint8_t)(int8_t)par << (8 * k);
+                }
+            }
+        }
+        uint64_t *dst = reinterpret_cast<uint64_t *>(wq8);
+        const long kk = (long)p.KH * p.KW * p.O_pad;
+        dst[(long)cbv * kk + ((long)ky * p.KW + kx) * p.O_pad + o] = vals;
+        dst[(long)(p.CBV + cbv) * kk + ((long)ky * p.KW + kx) * p.O_pad + o] = pars;
+    }
+}
+
+// One wave computes a 64 (channels) x 64 (pixels) tile with four 32x32x16 int8 MFMAs per step.
+// A step covers 16 reduction entries: one (ky,kx) tap of a PAIR of 8-channel blocks; lanes 0..31
+// feed block 2*cbp, lanes 32..63 block 2*cbp+1 (the MFMA's k = 8*(lane/32) + byte).
+constexpr int FT = 64;
+__global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restrict__ xq8, const int8_t *__restrict__ wq8,
+                                                         int32_t *__restrict__ out, Fixed8Params p)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int o_tiles = p.O_pad / FT;
+    const long tile = (long)blockIdx.x * 4 + wave;
+    const long m_tiles = (p.M + FT - 1) / FT;
+    if (tile >= m_tiles * o_tiles) return;
+    const int otile = (int)(tile % o_tiles);
+    const long mtile = tile / o_tiles;
+    const int j = lane & 31, h = lane >> 5;
+    const long plane = (long)p.Hp * p.Wp;
+
+    // the two pixel columns of this lane (pixel blocks 0 and 1 of the tile)
+    long xoff[2];
+    int mm[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+        long m = mtile * FT + pb * 32 + j;
+        mm[pb] = (int)(m < p.M ? m : p.M - 1);
+        const int n = mm[pb] / (p.Ho * p.Wo), r = mm[pb] - n * (p.Ho * p.Wo);
+        const int yo = r / p.Wo, xo = r - yo * p.Wo;
+        xoff[pb] = (long)n * p.CB * plane + (long)(yo * p.s0) * p.Wp + xo * p.s1;
+        if (m >= p.M) mm[pb] = -1;
+    }
+    const uint64_t *xb = reinterpret_cast<const uint64_t *>(xq8);
+    const uint64_t *wb = reinterpret_cast<const uint64_t *>(wq8);
+    const long wkk = (long)p.KH * p.KW * p.O_pad;
+
+    v16i acc[2][2]; // [channel block][pixel block]
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
+
+    for (int cbp = 0; cbp < p.CB / 2; cbp++) {
+        const int cb = 2 * cbp + h;
+        const uint64_t *xc = xb + (long)cb * plane;
+        const uint64_t *wc = wb + (long)cb * wkk + otile * FT + j;
+        for (int ky = 0; ky < p.KH; ky++)
+            for (int kx = 0; kx < p.KW; kx++) {
+                const long tap = (long)ky * p.Wp + kx;
+                const long b0 = (long)xc[xoff[0] + tap], b1 = (long)xc[xoff[1] + tap];
+                const uint64_t *wt = wc + ((long)ky * p.KW + kx) * p.O_pad;
+                const long a0 = (long)wt[0], a1 = (long)wt[32];
+                acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a0, b0, acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a0, b1, acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a1, b0, acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a1, b1, acc[1][1], 0, 0, 0);
+            }
+    }
+    // D[i][j]: column j = lane%32, row i = 8*(r/4) + 4*(lane/32) + r%4
+    const int HoWo = p.Ho * p.Wo;
+#pragma unroll
+    for (int pb = 0; pb < 2; pb++) {
+        if (mm[pb] < 0) continue;
+        const int n = mm[pb] / HoWo, r0 = mm[pb] - n * HoWo;
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int o = otile * FT + a * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+                if (o < p.O) out[((long)n * p.O + o) * HoWo + r0] = acc[a][pb][r];
+            }
+    }
+}
+
+// The MFMA path is exact only where the per-product saturating add is provably inert.
+static bool fixed_use_mfma(const FixedParams &p)
+{
+    if (p.add_config != 0 || p.d != 0 || p.pin > 7) return false;
+    const long pm = (1L << p.pin) - 1;
+    const long bound = (long)p.C * p.KH * p.KW * (pm * pm + 1); // largest possible rounded sum of one polarity
+    return bound < (long)p.max_value + 1 && (long)p.N * p.Ho * p.Wo < (1L << 31);
+}
+
 static int fixed_plan(const rexsc_fixed_desc *d, FixedParams &p, size_t &off_w, size_t &total)
 {
     REXSC_CHECK_ARG(d != nullptr, "null descriptor");
@@ -161,8 +330,14 @@ static int fixed_plan(const rexsc_fixed_desc *d, FixedParams &p, size_t &off_w, 
     p.d = 2 * d->precision_in - d->precision_out; if (p.d < 0) p.d = 0; // :97
     p.max_value = (int)(((((unsigned)1 << pmax) - 1u) >> p.d) << p.d);  // :96,:98
     p.P2 = (float)(1 << d->precision_in);
-    const size_t xbytes = (size_t)p.N * p.C * p.H * p.W * 4;
-    const size_t wbytes = (size_t)p.O * p.C * p.KH * p.KW * 4;
+    size_t xbytes = (size_t)p.N * p.C * p.H * p.W * 4;
+    size_t wbytes = (size_t)p.O * p.C * p.KH * p.KW * 4;
+    if (fixed_use_mfma(p)) {
+        const int CBV = ceil_div(p.C, 8);
+        const int O_pad = (int)align_up((size_t)p.O, FT);
+        xbytes = (size_t)p.N * 2 * CBV * (p.H + 2 * p.pad_h) * (p.W + 2 * p.pad_w) * 8;
+        wbytes = (size_t)2 * CBV * p.KH * p.KW * O_pad * 8;
+    }
     off_w = align_up(xbytes, 256);
     total = off_w + align_up(wbytes, 256);
     return REXSC_OK;
@@ -190,6 +365,31 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
     if (!workspace || workspace_bytes < total) {
         set_error("fixed conv2d: workspace of %zu bytes needed, %zu given", total, workspace ? workspace_bytes : (size_t)0);
         return REXSC_ERR_WORKSPACE;
+    }
+    if (fixed_use_mfma(p)) {
+        Fixed8Params q;
+        q.N = p.N; q.C = p.C; q.H = p.H; q.W = p.W; q.O = p.O; q.KH = p.KH; q.KW = p.KW;
+        q.O_pad = (int)align_up((size_t)p.O, FT);
+        q.pad_h = p.pad_h; q.pad_w = p.pad_w; q.s0 = p.s0; q.s1 = p.s1;
+        q.Hp = p.H + 2 * p.pad_h; q.Wp = p.W + 2 * p.pad_w; q.Ho = p.Ho; q.Wo = p.Wo;
+        q.CBV = ceil_div(p.C, 8); q.CB = 2 * q.CBV; q.M = p.N * p.Ho * p.Wo; q.P2 = p.P2;
+        int8_t *xq8 = (int8_t *)workspace;
+        int8_t *wq8 = (int8_t *)workspace + off_w;
+        auto gridf = [](long n) { long b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b ? b : 1)); };
+        const double io_bytes = 4.0 * p.N * p.C * p.H * p.W + 4.0 * p.O * p.C * p.KH * p.KW + 4.0 * p.N * p.O * p.Ho * p.Wo;
+        {
+            ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 8.0 * q.N * q.CB * q.Hp * q.Wp, stream);
+            hipLaunchKernelGGL(fixed_pack_act8_kernel, dim3(gridf((long)q.N * q.CBV * q.Hp * q.Wp)), dim3(256), 0, stream,
+                               x, xq8, q);
+            hipLaunchKernelGGL(fixed_pack_w8_kernel, dim3(gridf((long)q.CBV * q.KH * q.KW * q.O_pad)), dim3(256), 0,
+                               stream, w, wq8, q);
+        }
+        REXSC_CHECK_HIP(hipGetLastError());
+        const long tiles = (long)ceil_div(q.M, FT) * (q.O_pad / FT);
+        ProfScope prof("fixed_conv_mfma", io_bytes, stream);
+        hipLaunchKernelGGL(fixed_mfma_kernel, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, stream, xq8, wq8, out, q);
+        REXSC_CHECK_HIP(hipGetLastError());
+        return REXSC_OK;
     }
     int32_t *xq = (int32_t *)workspace;
     int32_t *wq = (int32_t *)((uint8_t *)workspace + off_w);

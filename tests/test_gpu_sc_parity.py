@@ -148,3 +148,36 @@ def test_conv_rejects_bad_arguments():
     with pytest.raises(RuntimeError, match="HIP device"):
         sc_extension_cuda.conv2d_generic_general_split_acc(x.cpu(), w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1,
                                                            True, False)
+
+
+RANDOM_FIXED = [
+    # N, C, H, W, O, KH, KW, stride, padding, add_config, pin, pout
+    (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), 0, 5, 24),     # int8 MFMA closed form, ResNet-like
+    (1, 20, 9, 11, 70, 3, 3, (2, 1), (1, 0), 0, 5, 24),      # odd channels / outputs / strides
+    (3, 8, 12, 12, 130, 1, 1, (1, 1), (0, 0), 0, 6, 24),     # 1x1, three output tiles
+    (1, 33, 8, 8, 5, 5, 5, (1, 1), (2, 2), 0, 7, 31),        # 7-bit operands, 5x5
+    (2, 128, 28, 28, 128, 3, 3, (1, 1), (1, 1), 0, 5, 24),   # config-4 stage 2 at batch 2
+    (1, 512, 7, 7, 512, 3, 3, (1, 1), (1, 1), 0, 5, 24),     # config-4 stage 4 at batch 1
+    (1, 16, 8, 8, 8, 3, 3, (1, 1), (1, 1), 0, 5, 8, 0.1),    # d > 0: VALU closed form with rounding (sparse operands)
+    (1, 64, 6, 6, 4, 3, 3, (1, 1), (1, 1), 0, 6, 12, 0.06),  # clamp fires for some outputs: VALU closed form
+    (1, 6, 7, 7, 5, 3, 3, (1, 1), (1, 1), 1, 5, 24),         # OR adder, sequential
+    (1, 7, 6, 6, 4, 3, 3, (1, 1), (1, 1), 3, 5, 24),         # pairwise OR2 adder, odd product count
+]
+
+
+@pytest.mark.parametrize("cfg", RANDOM_FIXED, ids=lambda c: "_".join(str(v) for v in c).replace(" ", ""))
+def test_fixed_random_vs_oracle(cfg):
+    import fixed_extension_cuda
+    N, C, H, W, O, KH, KW, stride, pad, add, pin, pout = cfg[:12]
+    dens = cfg[12] if len(cfg) > 12 else 1.0
+    print("fixed random", cfg, flush=True)
+    rng = np.random.default_rng(hash(cfg) & 0xFFFF)
+    P2 = 1 << pin
+    x = (rng.integers(0, 2 * P2, size=(N, C, H, W)) / (2 * P2)).astype(np.float32)   # half-grid: exercises round()
+    w = (rng.integers(-2 * P2 + 1, 2 * P2, size=(O, C, KH, KW)) / (2 * P2)).astype(np.float32)
+    x *= rng.uniform(size=x.shape) < dens
+    w *= rng.uniform(size=w.shape) < dens
+    out = fixed_extension_cuda.conv2d_saturate_acc(_dev(x), _dev(w), add, pin, pout, pad, stride)
+    want = orc.conv2d_saturate(x, w, add, pin, pout, pad, stride)
+    assert out.shape == want.shape and np.abs(want).max() > 0
+    assert np.array_equal(out.cpu().numpy(), want)
