@@ -72,7 +72,11 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
-    ap.add_argument("--cpu-sample-batch", type=int, default=16)
+    ap.add_argument("--cpu-sample-batch", type=int, default=64)
+    ap.add_argument("--only-layer", default=None, metavar="C,H,O,K,S",
+                    help="run a single SC conv layer shape instead of the 19 (for per-kernel counter runs)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="run three 256 MiB device-to-device copies and exit (scales the rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the SC path has no collectives); use --gpus 1",
@@ -89,13 +93,23 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     L, OR_N, N = 32, 2, args.batch
+    if args.copy_probe:
+        a = torch.zeros(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        return 0
     _lib.check(_lib.lib().rexsc_init(None), "rexsc_init")
 
+    shapes = RESNET18_SC_LAYERS
+    if args.only_layer:
+        shapes = [tuple(int(v) for v in args.only_layer.split(","))]
     layers = []
-    for i, (C, H, O, K, s) in enumerate(RESNET18_SC_LAYERS):
+    for i, (C, H, O, K, s) in enumerate(shapes):
         x, w = make_conv_operands(torch, N, C, H, O, K, L, seed=500 + i)
         layers.append((x.to(dev).contiguous(memory_format=torch.channels_last), w.to(dev), K, s))
-    total_mac = sum(layer_macs(N, C, H, O, K, s) for (C, H, O, K, s) in RESNET18_SC_LAYERS)
+    total_mac = sum(layer_macs(N, C, H, O, K, s) for (C, H, O, K, s) in shapes)
 
     def step():
         for (x, w, K, s) in layers:
@@ -120,7 +134,11 @@ def main():
     roofline = {
         "bound": "valu", "kernel": dom_name,
         "achieved": achieved / 1e12, "peak": VALU_PEAK_LANEOPS / 1e12, "unit": "Tlane-op/s",
-        "frac": achieved / VALU_PEAK_LANEOPS, "traffic": None,
+        "frac": achieved / VALU_PEAK_LANEOPS,
+        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the stage-2
+        # 3x3 layer (profiles/sc_compute_3x3_c128_hbm_traffic.md): 48.9 MB read + 25.7 MB written
+        # against 56.4 MB algorithmic; at these rates the kernel is nowhere near the HBM roof.
+        "traffic": 74.6e6, "traffic_shape": "128->128 3x3 28x28 batch 64",
         "avg_launch_us": dom["total_ms"] * 1e3 / dom["calls"], "launches": dom["calls"],
         "all_compute_kernels_frac": comp_ops / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS,
         "whole_step_frac": (total_mac * L * 4 / 32) / sec / VALU_PEAK_LANEOPS,
@@ -132,8 +150,9 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": sec * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u32",
         "data": "synthetic",
-        "config": {"workload": "resnet18_sc_conv_forward: 19 SC conv layers (16 3x3 + 3 1x1), batch %d, OR-%d, "
-                               "%d-bit streams, channels_last, float in / int16 pos+neg out" % (N, OR_N, L),
+        "config": {"workload": ("resnet18_sc_conv_forward: 19 SC conv layers (16 3x3 + 3 1x1), batch %d, OR-%d, "
+                                "%d-bit streams, channels_last, float in / int16 pos+neg out" % (N, OR_N, L))
+                               if not args.only_layer else "single SC conv layer C,H,O,K,S=%s, batch %d" % (args.only_layer, N),
                    "batch": N, "bit_length": L, "or_n": OR_N, "images_per_s": N / sec},
         "roofline": roofline,
     }
