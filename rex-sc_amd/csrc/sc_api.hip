@@ -1,6 +1,7 @@
 // extern "C" entry points for SC conv2d and SC linear: validation, planning (chunk widths,
 // tiles, slot splits, workspace carving) and kernel sequencing.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "sc_compute.h"
@@ -158,8 +159,11 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
     int splits = 1;
     const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
-    if (pl.tuned && waves < 4L * TARGET_WAVES) {
-        splits = (int)((4L * TARGET_WAVES + waves - 1) / waves);
+    // REXSC_TUNE_ROUNDS (default 4): how many rounds of resident waves a launch should have
+    // before slots are split over blocks as well
+    static const int rounds = []() { const char *e = getenv("REXSC_TUNE_ROUNDS"); int v = e ? atoi(e) : 4; return v > 0 ? v : 4; }();
+    if (pl.tuned && waves < (long)rounds * TARGET_WAVES) {
+        splits = (int)(((long)rounds * TARGET_WAVES + waves - 1) / waves);
         if (splits > max_splits) splits = max_splits;
         if (splits > 8) splits = 8;
     }

@@ -319,8 +319,11 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                 if (out_neg) out_neg[idx] = vn;
                 if (out_diff) out_diff[idx] = (int16_t)(vp - vn);
             } else {
-                // partial sums of a global slot split: part[plane][split][o][m]; plane 1 only in WIDE mode
-                const long idx = ((long)split * p.O_pad + oo) * p.M + m;
+                // partial sums of a global slot split, laid out like the final tensor so that the
+                // finalize pass is coalesced on both sides: part[plane][split][o][m] for NCHW,
+                // part[plane][split][m][o] for NHWC; plane 1 only in WIDE mode
+                const long idx = p.out_channels_last ? ((long)split * p.M + m) * p.O_pad + oo
+                                                     : ((long)split * p.O_pad + oo) * p.M + m;
                 part[idx] = v;
                 if (WIDE) part[plane + idx] = vw;
             }
@@ -339,16 +342,21 @@ __global__ __launch_bounds__(256) void sc_finalize_kernel(const uint32_t *__rest
     const long total = (long)p.O * p.M;
     const long plane = (long)p.splits * p.O_pad * p.M;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-        const int o = (int)(i / p.M), m = (int)(i - (long)o * p.M);
+        // i runs in output memory order
+        int o, m;
+        if (p.out_channels_last) { m = (int)(i / p.O); o = (int)(i - (long)m * p.O); }
+        else {
+            const long no = i / p.HoWo; // n*O + o
+            const int r = (int)(i - no * p.HoWo), n = (int)(no / p.O);
+            o = (int)(no - (long)n * p.O); m = n * p.HoWo + r;
+        }
         uint32_t sp = 0, sn = 0;
         for (int s = 0; s < p.splits; s++) {
-            const long idx = ((long)s * p.O_pad + o) * p.M + m;
+            const long idx = p.out_channels_last ? ((long)s * p.M + m) * p.O_pad + o : ((long)s * p.O_pad + o) * p.M + m;
             if (WIDE) { sp += part[idx]; sn += part[plane + idx]; }
             else { const uint32_t v = part[idx]; sp += v & 0xffffu; sn += v >> 16; }
         }
-        long idx;
-        if (p.out_channels_last) idx = (long)m * p.O + o;
-        else { const int n = m / p.HoWo, r = m - n * p.HoWo; idx = ((long)n * p.O + o) * p.HoWo + r; }
+        const long idx = i;
         const OutT vp = (OutT)sp, vn = (OutT)sn; // int16: wraps
         if (out_pos) out_pos[idx] = vp;
         if (out_neg) out_neg[idx] = vn;

@@ -162,31 +162,49 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
 
     load_tables_to_lds(tables + seq_index(gp.lb, gp.acc), s_seq, s_inv);
 
-    // phase 1: load + quantise -> s_q[channel][pixel]
+    // phase 1: load + quantise -> s_q[channel][pixel].  All loads of a thread are issued before the
+    // first one is consumed (fully unrolled into registers): the phase costs one memory latency,
+    // not one per element.
     if (!geo.channels_last) {
+        // lane = pixel, the block's waves interleave over the channels of the chunk
         const int pp = pp0 + lane;
         const int yp = pp / geo.Wp, xp = pp - yp * geo.Wp;
         const int y = yp - geo.pad_h, xx = xp - geo.pad_w;
         const bool inb = (lane < npix) && y >= 0 && y < geo.H && xx >= 0 && xx < geo.W;
-        for (int cl = wave; cl < CCH; cl += 4) {
-            const int c = zg * CCH + cl;
-            int q = 0;
-            if (inb && c < geo.C) q = quant_ceil_pos(x[(((long)n * geo.C + c) * geo.H + y) * geo.W + xx], S);
-            s_q[cl * QPITCH + lane] = (uint8_t)q;
+        constexpr int PER = CCH / 4;
+        float v[PER];
+#pragma unroll
+        for (int k = 0; k < PER; k++) {
+            const int c = zg * CCH + wave + 4 * k;
+            v[k] = (inb && c < geo.C) ? x[(((long)n * geo.C + c) * geo.H + y) * geo.W + xx] : 0.f;
         }
+#pragma unroll
+        for (int k = 0; k < PER; k++) s_q[(wave + 4 * k) * QPITCH + lane] = (uint8_t)quant_ceil_pos(v[k], S);
     } else {
-        for (int j = wave; j < ACT_TILE; j += 4) {
+        // lane = channel, each wave takes 16 pixels
+        constexpr int PIX = ACT_TILE / 4, PASS = (CCH + 63) / 64;
+        float v[PIX][PASS];
+#pragma unroll
+        for (int k = 0; k < PIX; k++) {
+            const int j = wave + 4 * k;
             const int pp = pp0 + j;
             const int yp = pp / geo.Wp, xp = pp - yp * geo.Wp;
             const int y = yp - geo.pad_h, xx = xp - geo.pad_w;
             const bool inb = (j < npix) && y >= 0 && y < geo.H && xx >= 0 && xx < geo.W;
-            for (int cl = lane; cl < CCH; cl += 64) {
+#pragma unroll
+            for (int h = 0; h < PASS; h++) {
+                const int cl = h * 64 + lane;
                 const int c = zg * CCH + cl;
-                int q = 0;
-                if (inb && c < geo.C) q = quant_ceil_pos(x[(((long)n * geo.H + y) * geo.W + xx) * geo.C + c], S);
-                s_q[cl * QPITCH + j] = (uint8_t)q;
+                v[k][h] = (inb && cl < CCH && c < geo.C) ? x[(((long)n * geo.H + y) * geo.W + xx) * geo.C + c] : 0.f;
             }
         }
+#pragma unroll
+        for (int k = 0; k < PIX; k++)
+#pragma unroll
+            for (int h = 0; h < PASS; h++) {
+                const int cl = h * 64 + lane;
+                if (cl < CCH) s_q[cl * QPITCH + wave + 4 * k] = (uint8_t)quant_ceil_pos(v[k][h], S);
+            }
     }
     __syncthreads();
 
@@ -235,14 +253,15 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
 
 // ---- weight SNG ------------------------------------------------------------------------------
 // Output layout: Wst[slot][ky][zg][o][pol][kx][zc]  (o padded to O_pad; padded rows are zero).
-// Block: 256 threads, one (o-group of W_OG, ky, zg).
-constexpr int W_OG = 16;
+// Block: 256 threads, one (group of `wog` output channels, ky, zg); wog is 16, 8, 4 or 2, the largest
+// that still gives the launch a few thousand blocks.
+constexpr int W_OG_MAX = 16;
 constexpr int W_SLOT_GROUP = 32; // upper bound; the launcher shrinks it to fit the LDS budget
 
 template <int ZC>
 __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict__ w, uint32_t *__restrict__ Wst,
                                                          const SeqTable *__restrict__ tables, WeightGeom geo, GenParams gp,
-                                                         int slot_group)
+                                                         int slot_group, int wog)
 {
     constexpr int CCH = 32 * ZC;
     constexpr int HALVES = (CCH + 63) / 64;
@@ -254,31 +273,41 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int og = blockIdx.x, ky = blockIdx.y, zg = blockIdx.z;
     const int KW = geo.KW;
-    const int row = W_OG * 2 * KW * ZC; // words per slot handled by this block
+    const int row = wog * 2 * KW * ZC; // words per slot handled by this block
     const int pitch = row + 2;          // LDS row pitch (bank spreading for the per-slot writes)
     const float S = (float)gp.scale;
 
     load_tables_to_lds(tables + seq_index(gp.lb, gp.acc), s_seq, s_inv);
     __syncthreads();
 
-    const int ntask = W_OG * KW * HALVES;
+    const int ntask = wog * KW * HALVES;
+    auto task_weight = [&](int task) -> float {
+        const int h = task % HALVES;
+        const int kx = (task / HALVES) % KW;
+        const int ol = task / (HALVES * KW);
+        const int o = og * wog + ol;
+        const int cl = h * 64 + lane;
+        const int c = zg * CCH + cl;
+        if (task < ntask && cl < CCH && c < geo.C && o < geo.O) {
+            const long wi = geo.channels_last ? (((long)o * geo.KH + ky) * KW + kx) * geo.C + c
+                                              : (((long)o * geo.C + c) * geo.KH + ky) * KW + kx;
+            return w[wi];
+        }
+        return 0.f;
+    };
+
     for (int s0 = 0; s0 < gp.n_slots; s0 += slot_group) {
         const int ns = min(slot_group, gp.n_slots - s0);
+        float f = task_weight(wave);
         for (int task = wave; task < ntask; task += 4) {
+            const float f_next = task_weight(task + 4); // in flight while this task's slots are generated
             const int h = task % HALVES;
             const int kx = (task / HALVES) % KW;
             const int ol = task / (HALVES * KW);
-            const int o = og * W_OG + ol;
             const int cl = h * 64 + lane;
             const int c = zg * CCH + cl;
-            int vp = 0, vn = 0;
-            if (cl < CCH && c < geo.C && o < geo.O) {
-                long wi = geo.channels_last ? (((long)o * geo.KH + ky) * KW + kx) * geo.C + c
-                                            : (((long)o * geo.C + c) * geo.KH + ky) * KW + kx;
-                const float f = w[wi];
-                vp = quant_ceil_pos(f, S);
-                vn = quant_ceil_neg(f, S);
-            }
+            const int vp = quant_ceil_pos(f, S);
+            const int vn = quant_ceil_neg(f, S);
             // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
             const int sd = (int)((13L + (long)c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
             const int pos = s_inv[sd + 1] + 1;
@@ -291,10 +320,11 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
                 dp[0] = plo; dn[0] = nlo;
                 if (ZC > 1) { dp[1] = phi; dn[1] = nhi; }
             }
+            f = f_next;
         }
         __syncthreads();
         for (int s = 0; s < ns; s++) {
-            uint32_t *dst = Wst + ((((long)(s0 + s) * geo.KH + ky) * geo.ZG + zg) * geo.O_pad + og * W_OG) * 2 * KW * ZC;
+            uint32_t *dst = Wst + ((((long)(s0 + s) * geo.KH + ky) * geo.ZG + zg) * geo.O_pad + og * wog) * 2 * KW * ZC;
             for (int i = tid; i < row; i += 256) dst[i] = s_stage[s * pitch + i];
         }
         __syncthreads();
@@ -333,15 +363,17 @@ template <int ZC>
 static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, const WeightGeom &geo,
                          const GenParams &gp, hipStream_t stream)
 {
-    dim3 grid(geo.O_pad / W_OG, geo.KH, geo.ZG);
-    const size_t row_bytes = sizeof(uint32_t) * (W_OG * 2 * geo.KW * ZC + 2);
+    int wog = W_OG_MAX;
+    while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < 2048) wog /= 2;
+    dim3 grid(geo.O_pad / wog, geo.KH, geo.ZG);
+    const size_t row_bytes = sizeof(uint32_t) * (wog * 2 * geo.KW * ZC + 2);
     int slot_group = (int)((60 * 1024 - SEQ_LEN - 256) / row_bytes);
     if (slot_group > W_SLOT_GROUP) slot_group = W_SLOT_GROUP;
     REXSC_CHECK_ARG(slot_group >= 1, "weight SNG: kernel width %d too large for LDS staging", geo.KW);
     const size_t lds = SEQ_LEN + 256 + row_bytes * slot_group;
     ProfScope prof("sng_weight", 4.0 * geo.O * geo.C * geo.KH * geo.KW +
                                      4.0 * gp.n_slots * geo.KH * geo.ZG * geo.O_pad * 2 * geo.KW * ZC, stream);
-    hipLaunchKernelGGL(sng_weight_kernel<ZC>, grid, dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group);
+    hipLaunchKernelGGL(sng_weight_kernel<ZC>, grid, dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group, wog);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
@@ -351,7 +383,7 @@ int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenP
     const SeqTable *tables = nullptr;
     int rc = get_seq_tables(&tables, stream);
     if (rc) return rc;
-    REXSC_CHECK_ARG(geo.O_pad % W_OG == 0, "weight SNG: O_pad %d not a multiple of %d", geo.O_pad, W_OG);
+    REXSC_CHECK_ARG(geo.O_pad % W_OG_MAX == 0, "weight SNG: O_pad %d not a multiple of %d", geo.O_pad, W_OG_MAX);
     REXSC_CHECK_ARG(geo.KH <= 65535 && geo.ZG <= 65535, "weight SNG: grid too large");
     switch (geo.ZC) {
     case 1: return launch_weight<1>(w, Wst, tables, geo, gp, stream);
