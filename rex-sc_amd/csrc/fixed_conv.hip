@@ -144,122 +144,135 @@ __global__ __launch_bounds__(256) void fixed_conv_kernel(const int32_t *__restri
 
 // ---- int8 MFMA path for the closed form ----------------------------------------------------------
 // Valid when add_config = 0, d = 0, operands fit int8 (precision_in <= 7) and the clamp cannot fire
-// (C*KH*KW*((2^pin-1)^2+1) < max_value+1).  Then pos - neg collapses to ONE signed contraction with
-// the reduction doubled:  out = sum a*w  +  sum (a&1) * sgn(w)*(|w|&1).
+// (C*KH*KW*((2^pin-1)^2+1) < max_value+1).  Then pos - neg collapses to ONE signed contraction plus
+// a parity term:   out = sum a*w  +  sum (a&1) * sgn(w)*(|w|&1).
 //
-// Operands are re-laid-out once, channel-blocked by 8 so that every MFMA operand fetch is an
-// 8-byte load and adjacent lanes read adjacent memory:
-//   xq8[n][cb][yp][xp][8]   int8, zero padded plane; blocks [0,CBV) values, [CBV,2*CBV) parities
-//   wq8[cb][ky][kx][o_pad][8] int8, same block order
-// GEMM orientation: MFMA rows = output channels (weights are the A operand), MFMA columns =
-// pixels (activations are the B operand), so that the 32 lanes of a half-wave hold 32
-// consecutive pixels of one output channel and the int32 NCHW stores are 128-byte runs.
+// Operands are re-laid-out once, channel-blocked by 16 so that every MFMA operand fetch is one
+// 16-byte load and adjacent lanes read adjacent memory:
+//   xq16[n][cb][yp][xp][16]     int8 activations over the zero-padded plane
+//   wq16[cb][ky][kx][o_pad][16] int8 signed weights;  wp16 (same shape) = sgn(w)*(|w|&1)
+// The activation parities are not stored: a&1 is one v_and on the loaded bytes.
+// GEMM orientation: MFMA rows = output channels (weights are the A operand), MFMA columns = pixels
+// (activations are the B operand): the 32 lanes of a half-wave hold 32 consecutive pixels of one
+// output channel, so the int32 NCHW stores are 128-byte runs.
+// v_mfma_i32_32x32x32_i8: lane l feeds row/column l%32 with k = 16*(l/32) .. +15, i.e. the two
+// half-waves take two consecutive 16-channel blocks; D[i][j] sits in lane (j + 32*((i/4)%2)),
+// register 4*(i/8) + i%4.
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef int v4i __attribute__((ext_vector_type(4)));
 
 struct Fixed8Params {
     int N, C, H, W, O, O_pad, KH, KW;
     int pad_h, pad_w, s0, s1, Hp, Wp, Ho, Wo;
-    int CBV, CB; // value blocks, total blocks (= 2*CBV)
+    int CB;      // 16-channel blocks, padded to an even count
     int M;       // N*Ho*Wo
+    int ksplit;  // blocks of the reduction handled by different waves (results added atomically)
     float P2;
 };
 
-__global__ __launch_bounds__(256) void fixed_pack_act8_kernel(const float *__restrict__ x, int8_t *__restrict__ xq8,
-                                                              Fixed8Params p)
+__global__ __launch_bounds__(256) void fixed_pack_act16_kernel(const float *__restrict__ x, int8_t *__restrict__ xq16,
+                                                               Fixed8Params p)
 {
-    // one thread per (n, cbv, yp, xp): 8 channels -> one value block and one parity block
-    const long total = (long)p.N * p.CBV * p.Hp * p.Wp;
+    // one thread per (n, cb, yp, xp): 16 channels -> 16 bytes
+    const long total = (long)p.N * p.CB * p.Hp * p.Wp;
     const long stride = (long)gridDim.x * blockDim.x;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
         const int xp = (int)(i % p.Wp);
         const int yp = (int)((i / p.Wp) % p.Hp);
-        const int cbv = (int)((i / ((long)p.Wp * p.Hp)) % p.CBV);
-        const int n = (int)(i / ((long)p.Wp * p.Hp * p.CBV));
+        const int cb = (int)((i / ((long)p.Wp * p.Hp)) % p.CB);
+        const int n = (int)(i / ((long)p.Wp * p.Hp * p.CB));
         const int y = yp - p.pad_h, xx = xp - p.pad_w;
         const bool inb = y >= 0 && y < p.H && xx >= 0 && xx < p.W;
-        uint64_t vals = 0, pars = 0;
-        if (inb) {
+        float f[16];
 #pragma unroll
-            for (int k = 0; k < 8; k++) {
-                const int c = cbv * 8 + k;
-                if (c < p.C) {
-                    const int q = quant_round_pos(x[(((long)n * p.C + c) * p.H + y) * p.W + xx], p.P2);
-                    vals |= (uint64_t)(uint8_t)q << (8 * k);
-                    pars |= (uint64_t)(q & 1) << (8 * k);
-                }
-            }
+        for (int k = 0; k < 16; k++) {
+            const int c = cb * 16 + k;
+            f[k] = (inb && c < p.C) ? x[(((long)n * p.C + c) * p.H + y) * p.W + xx] : 0.f;
         }
-        const long plane = (long)p.Hp * p.Wp;
-        uint64_t *dst = reinterpret_cast<uint64_t *>(xq8);
-        dst[((long)n * p.CB + cbv) * plane + (long)yp * p.Wp + xp] = vals;
-        dst[((long)n * p.CB + p.CBV + cbv) * plane + (long)yp * p.Wp + xp] = pars;
+        uint32_t wds[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < 16; k++) wds[k >> 2] |= (uint32_t)(uint8_t)quant_round_pos(f[k], p.P2) << (8 * (k & 3));
+        reinterpret_cast<uint4 *>(xq16)[i] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
     }
 }
 
-__global__ __launch_bounds__(256) void fixed_pack_w8_kernel(const float *__restrict__ w, int8_t *__restrict__ wq8,
-                                                            Fixed8Params p)
+__global__ __launch_bounds__(256) void fixed_pack_w16_kernel(const float *__restrict__ w, int8_t *__restrict__ wq16,
+                                                             int8_t *__restrict__ wp16, Fixed8Params p)
 {
-    const long total = (long)p.CBV * p.KH * p.KW * p.O_pad;
+    const long total = (long)p.CB * p.KH * p.KW * p.O_pad;
     const long stride = (long)gridDim.x * blockDim.x;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
         const int o = (int)(i % p.O_pad);
         const int kx = (int)((i / p.O_pad) % p.KW);
         const int ky = (int)((i / ((long)p.O_pad * p.KW)) % p.KH);
-        const int cbv = (int)(i / ((long)p.O_pad * p.KW * p.KH));
-        uint64_t vals = 0, pars = 0;
+        const int cb = (int)(i / ((long)p.O_pad * p.KW * p.KH));
+        uint32_t vals[4] = {0, 0, 0, 0}, pars[4] = {0, 0, 0, 0};
         if (o < p.O) {
 #pragma unroll
-            for (int k = 0; k < 8; k++) {
-                const int c = cbv * 8 + k;
+            for (int k = 0; k < 16; k++) {
+                const int c = cb * 16 + k;
                 if (c < p.C) {
                     const float f = w[(((long)o * p.C + c) * p.KH + ky) * p.KW + kx];
                     const int q = quant_round_pos(f, p.P2) - quant_round_neg(f, p.P2); // signed
                     const int par = (q & 1) ? (q < 0 ? -1 : 1) : 0;
-                    vals |= (uint64_t)(uint8_t)(int8_t)q << (8 * k);
-                    pars |= (uint64_t)(uint8_t)(int8_t)par << (8 * k);
+                    vals[k >> 2] |= (uint32_t)(uint8_t)(int8_t)q << (8 * (k & 3));
+                    pars[k >> 2] |= (uint32_t)(uint8_t)(int8_t)par << (8 * (k & 3));
                 }
             }
         }
-        uint64_t *dst = reinterpret_cast<uint64_t *>(wq8);
-        const long kk = (long)p.KH * p.KW * p.O_pad;
-        dst[(long)cbv * kk + ((long)ky * p.KW + kx) * p.O_pad + o] = vals;
-        dst[(long)(p.CBV + cbv) * kk + ((long)ky * p.KW + kx) * p.O_pad + o] = pars;
+        reinterpret_cast<uint4 *>(wq16)[i] = make_uint4(vals[0], vals[1], vals[2], vals[3]);
+        reinterpret_cast<uint4 *>(wp16)[i] = make_uint4(pars[0], pars[1], pars[2], pars[3]);
     }
 }
 
-// One wave computes a 64 (channels) x 64 (pixels) tile with four 32x32x16 int8 MFMAs per step.
-// A step covers 16 reduction entries: one (ky,kx) tap of a PAIR of 8-channel blocks; lanes 0..31
-// feed block 2*cbp, lanes 32..63 block 2*cbp+1 (the MFMA's k = 8*(lane/32) + byte).
-constexpr int FT = 64;
-__global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restrict__ xq8, const int8_t *__restrict__ wq8,
-                                                         int32_t *__restrict__ out, Fixed8Params p)
+__global__ void fixed_zero_kernel(int32_t *__restrict__ p, size_t n)
 {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
+}
+
+// A block of 4 waves computes a 64 (channels) x 256 (pixels) tile over its share of the channel-block
+// pairs; each wave owns 64 pixels.  The weights of one pair (both half-wave blocks, all taps, values
+// and parities) are staged in LDS once per block and read with ds_read_b128, so they cost L2
+// bandwidth once per 256 pixels instead of once per 64.  Per kernel row all KW taps are loaded
+// first, then the 8*KW MFMAs run: one exposed memory latency per row instead of one per tap.
+constexpr int FT = 64;
+template <int KW>
+__global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restrict__ xq16, const int8_t *__restrict__ wq16,
+                                                         const int8_t *__restrict__ wp16, int32_t *__restrict__ out,
+                                                         Fixed8Params p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_raw[];
+    v4i *s_w = reinterpret_cast<v4i *>(s_raw); // [h][tap][val/par][o 0..63]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int o_tiles = p.O_pad / FT;
-    const long tile = (long)blockIdx.x * 4 + wave;
     const long m_tiles = (p.M + FT - 1) / FT;
-    if (tile >= m_tiles * o_tiles) return;
-    const int otile = (int)(tile % o_tiles);
-    const long mtile = tile / o_tiles;
+    const long m_groups = (m_tiles + 3) / 4;
+    long blk = blockIdx.x;
+    const int ks = (int)(blk % p.ksplit); blk /= p.ksplit;
+    const int otile = (int)(blk % o_tiles);
+    const long mtile = (blk / o_tiles) * 4 + wave;   // may be past the end: such a wave only helps staging
+    (void)m_groups;
     const int j = lane & 31, h = lane >> 5;
     const long plane = (long)p.Hp * p.Wp;
+    const int taps = p.KH * KW;
 
-    // the two pixel columns of this lane (pixel blocks 0 and 1 of the tile)
     long xoff[2];
     int mm[2];
 #pragma unroll
     for (int pb = 0; pb < 2; pb++) {
-        long m = mtile * FT + pb * 32 + j;
+        const long m = mtile * FT + pb * 32 + j;
         mm[pb] = (int)(m < p.M ? m : p.M - 1);
         const int n = mm[pb] / (p.Ho * p.Wo), r = mm[pb] - n * (p.Ho * p.Wo);
         const int yo = r / p.Wo, xo = r - yo * p.Wo;
         xoff[pb] = (long)n * p.CB * plane + (long)(yo * p.s0) * p.Wp + xo * p.s1;
         if (m >= p.M) mm[pb] = -1;
     }
-    const uint64_t *xb = reinterpret_cast<const uint64_t *>(xq8);
-    const uint64_t *wb = reinterpret_cast<const uint64_t *>(wq8);
-    const long wkk = (long)p.KH * p.KW * p.O_pad;
+    const v4i *xb = reinterpret_cast<const v4i *>(xq16);
+    const v4i *wb = reinterpret_cast<const v4i *>(wq16);
+    const v4i *wpb = reinterpret_cast<const v4i *>(wp16);
+    const long wkk = (long)taps * p.O_pad;
 
     v16i acc[2][2]; // [channel block][pixel block]
 #pragma unroll
@@ -269,23 +282,58 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
 
-    for (int cbp = 0; cbp < p.CB / 2; cbp++) {
-        const int cb = 2 * cbp + h;
-        const uint64_t *xc = xb + (long)cb * plane;
-        const uint64_t *wc = wb + (long)cb * wkk + otile * FT + j;
-        for (int ky = 0; ky < p.KH; ky++)
-            for (int kx = 0; kx < p.KW; kx++) {
-                const long tap = (long)ky * p.Wp + kx;
-                const long b0 = (long)xc[xoff[0] + tap], b1 = (long)xc[xoff[1] + tap];
-                const uint64_t *wt = wc + ((long)ky * p.KW + kx) * p.O_pad;
-                const long a0 = (long)wt[0], a1 = (long)wt[32];
-                acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a0, b0, acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a0, b1, acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a1, b0, acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x16_i8(a1, b1, acc[1][1], 0, 0, 0);
-            }
+    const int pairs = p.CB / 2;
+    const int per = (pairs + p.ksplit - 1) / p.ksplit;
+    const int cbp_begin = ks * per, cbp_end = min(pairs, cbp_begin + per);
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    // Activation rows are software-pipelined: the KW taps of the next (pair, ky) row are requested
+    // before the MFMAs of the current row are issued.
+    v4i b0[KW], b1[KW], n0[KW], n1[KW];
+    if (cbp_begin < cbp_end) {
+        const v4i *xc = xb + (long)(2 * cbp_begin + h) * plane;
+#pragma unroll
+        for (int kx = 0; kx < KW; kx++) { b0[kx] = xc[xoff[0] + kx]; b1[kx] = xc[xoff[1] + kx]; }
     }
-    // D[i][j]: column j = lane%32, row i = 8*(r/4) + 4*(lane/32) + r%4
+    for (int cbp = cbp_begin; cbp < cbp_end; cbp++) {
+        // stage the pair's weights: 2 (h) x taps x 2 (val, par) x 64 (o) 16-byte entries
+        __syncthreads();
+        for (int e = threadIdx.x; e < 2 * taps * 2 * FT; e += 256) {
+            const int o = e % FT, vp = (e / FT) % 2, tap = (e / (2 * FT)) % taps, hh = e / (2 * FT * taps);
+            const long src = (long)(2 * cbp + hh) * wkk + (long)tap * p.O_pad + otile * FT + o;
+            s_w[e] = vp ? wpb[src] : wb[src];
+        }
+        __syncthreads();
+        const v4i *sw = s_w + (long)h * taps * 2 * FT + j;
+        for (int ky = 0; ky < p.KH; ky++) {
+            {
+                // next row: (cbp, ky+1), or row 0 of the next pair; the very last row re-reads itself
+                int cn = cbp, kn = ky + 1;
+                if (kn == p.KH) { kn = 0; cn = cbp + 1; }
+                if (cn >= cbp_end) { cn = cbp; kn = ky; }
+                const v4i *xn = xb + (long)(2 * cn + h) * plane + (long)kn * p.Wp;
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++) { n0[kx] = xn[xoff[0] + kx]; n1[kx] = xn[xoff[1] + kx]; }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) {
+                const v4i *wt = sw + (ky * KW + kx) * 2 * FT;
+                const v4i a0 = wt[0], a1 = wt[32], q0 = wt[FT], q1 = wt[FT + 32];
+                const v4i p0 = b0[kx] & ones, p1 = b1[kx] & ones; // activation parities
+                acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0[kx], acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b1[kx], acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b0[kx], acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1[kx], acc[1][1], 0, 0, 0);
+                acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, p0, acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, p1, acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, p0, acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, p1, acc[1][1], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) { b0[kx] = n0[kx]; b1[kx] = n1[kx]; }
+        }
+    }
     const int HoWo = p.Ho * p.Wo;
 #pragma unroll
     for (int pb = 0; pb < 2; pb++) {
@@ -296,7 +344,10 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int o = otile * FT + a * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-                if (o < p.O) out[((long)n * p.O + o) * HoWo + r0] = acc[a][pb][r];
+                if (o >= p.O) continue;
+                int32_t *dst = out + ((long)n * p.O + o) * HoWo + r0;
+                if (p.ksplit == 1) *dst = acc[a][pb][r];
+                else atomicAdd(dst, acc[a][pb][r]); // integer adds commute: the split is exact
             }
     }
 }
@@ -305,6 +356,8 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
 static bool fixed_use_mfma(const FixedParams &p)
 {
     if (p.add_config != 0 || p.d != 0 || p.pin > 7) return false;
+    if (p.KW != 1 && p.KW != 3 && p.KW != 5) return false; // unrolled instances of the MFMA kernel
+    if ((long)p.KH * p.KW * 4096 > 60 * 1024) return false;   // weight staging must fit the default LDS window
     const long pm = (1L << p.pin) - 1;
     const long bound = (long)p.C * p.KH * p.KW * (pm * pm + 1); // largest possible rounded sum of one polarity
     return bound < (long)p.max_value + 1 && (long)p.N * p.Ho * p.Wo < (1L << 31);
@@ -333,10 +386,10 @@ static int fixed_plan(const rexsc_fixed_desc *d, FixedParams &p, size_t &off_w, 
     size_t xbytes = (size_t)p.N * p.C * p.H * p.W * 4;
     size_t wbytes = (size_t)p.O * p.C * p.KH * p.KW * 4;
     if (fixed_use_mfma(p)) {
-        const int CBV = ceil_div(p.C, 8);
+        const int CB = (int)align_up((size_t)ceil_div(p.C, 16), 2);
         const int O_pad = (int)align_up((size_t)p.O, FT);
-        xbytes = (size_t)p.N * 2 * CBV * (p.H + 2 * p.pad_h) * (p.W + 2 * p.pad_w) * 8;
-        wbytes = (size_t)2 * CBV * p.KH * p.KW * O_pad * 8;
+        xbytes = (size_t)p.N * CB * (p.H + 2 * p.pad_h) * (p.W + 2 * p.pad_w) * 16;
+        wbytes = 2 * (size_t)CB * p.KH * p.KW * O_pad * 16; // values + parities
     }
     off_w = align_up(xbytes, 256);
     total = off_w + align_up(wbytes, 256);
@@ -372,22 +425,37 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         q.O_pad = (int)align_up((size_t)p.O, FT);
         q.pad_h = p.pad_h; q.pad_w = p.pad_w; q.s0 = p.s0; q.s1 = p.s1;
         q.Hp = p.H + 2 * p.pad_h; q.Wp = p.W + 2 * p.pad_w; q.Ho = p.Ho; q.Wo = p.Wo;
-        q.CBV = ceil_div(p.C, 8); q.CB = 2 * q.CBV; q.M = p.N * p.Ho * p.Wo; q.P2 = p.P2;
-        int8_t *xq8 = (int8_t *)workspace;
-        int8_t *wq8 = (int8_t *)workspace + off_w;
-        auto gridf = [](long n) { long b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : (b ? b : 1)); };
-        const double io_bytes = 4.0 * p.N * p.C * p.H * p.W + 4.0 * p.O * p.C * p.KH * p.KW + 4.0 * p.N * p.O * p.Ho * p.Wo;
+        q.CB = (int)align_up((size_t)ceil_div(p.C, 16), 2); q.M = p.N * p.Ho * p.Wo; q.P2 = p.P2;
+        // split the channel-block pairs over waves until the launch has a few thousand of them
+        const long tiles = (long)ceil_div(q.M, FT) * (q.O_pad / FT);
+        q.ksplit = 1;
+        while (tiles * q.ksplit < 3072 && q.ksplit * 2 <= q.CB / 2) q.ksplit *= 2;
+        int8_t *xq16 = (int8_t *)workspace;
+        int8_t *wq16 = (int8_t *)workspace + off_w;
+        int8_t *wp16 = wq16 + (size_t)q.CB * q.KH * q.KW * q.O_pad * 16;
+        auto gridf = [](long n) { long b = (n + 255) / 256; return (int)(b > 16384 ? 16384 : (b ? b : 1)); };
+        const size_t nout = (size_t)p.N * p.O * p.Ho * p.Wo;
+        const double io_bytes = 4.0 * p.N * p.C * p.H * p.W + 4.0 * p.O * p.C * p.KH * p.KW + 4.0 * nout;
         {
-            ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 8.0 * q.N * q.CB * q.Hp * q.Wp, stream);
-            hipLaunchKernelGGL(fixed_pack_act8_kernel, dim3(gridf((long)q.N * q.CBV * q.Hp * q.Wp)), dim3(256), 0, stream,
-                               x, xq8, q);
-            hipLaunchKernelGGL(fixed_pack_w8_kernel, dim3(gridf((long)q.CBV * q.KH * q.KW * q.O_pad)), dim3(256), 0,
-                               stream, w, wq8, q);
+            ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 16.0 * q.N * q.CB * q.Hp * q.Wp, stream);
+            hipLaunchKernelGGL(fixed_pack_act16_kernel, dim3(gridf((long)q.N * q.CB * q.Hp * q.Wp)), dim3(256), 0, stream,
+                               x, xq16, q);
+            hipLaunchKernelGGL(fixed_pack_w16_kernel, dim3(gridf((long)q.CB * q.KH * q.KW * q.O_pad)), dim3(256), 0,
+                               stream, w, wq16, wp16, q);
+            if (q.ksplit > 1)
+                hipLaunchKernelGGL(fixed_zero_kernel, dim3(gridf((long)nout / 4 + 1)), dim3(256), 0, stream, out, nout);
         }
         REXSC_CHECK_HIP(hipGetLastError());
-        const long tiles = (long)ceil_div(q.M, FT) * (q.O_pad / FT);
+        const long m_groups = ((long)ceil_div(q.M, FT) + 3) / 4;
+        const unsigned grid = (unsigned)(m_groups * (q.O_pad / FT) * q.ksplit);
+        const size_t lds = (size_t)2 * q.KH * q.KW * 2 * FT * 16;
         ProfScope prof("fixed_conv_mfma", io_bytes, stream);
-        hipLaunchKernelGGL(fixed_mfma_kernel, dim3((unsigned)((tiles + 3) / 4)), dim3(256), 0, stream, xq8, wq8, out, q);
+        switch (q.KW) {
+        case 1: hipLaunchKernelGGL(fixed_mfma_kernel<1>, dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q); break;
+        case 3: hipLaunchKernelGGL(fixed_mfma_kernel<3>, dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q); break;
+        case 5: hipLaunchKernelGGL(fixed_mfma_kernel<5>, dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q); break;
+        default: break; // excluded by fixed_use_mfma
+        }
         REXSC_CHECK_HIP(hipGetLastError());
         return REXSC_OK;
     }
