@@ -62,6 +62,12 @@ typedef struct rexsc_conv_desc {
 
 size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d);
 
+/* Planning decisions for a descriptor (no counterpart in the reference; for tests and tuning):
+ * out[0..15] = {tuned kernel?, KW, words per chunk, chunks, O padded, pixels per lane, waves per
+ * block, slot splits, slots per split, slots, direct store?, images per batch chunk, output pixels
+ * per chunk, padded H, padded W, wide accumulators?}. */
+int rexsc_conv2d_plan_info(const rexsc_conv_desc *d, int64_t *out);
+
 /* x, w: float32 device arrays in the memory order the descriptor states.
  * out_pos, out_neg: int16 [N][O][Ho][Wo] (or NHWC), Ho=(H+2*pad_h-KH)/stride_h+1.
  * Either output pointer may be NULL together with out_diff != NULL to get pos-neg (int16,

@@ -282,7 +282,11 @@ int orc_linear(const int32_t *xq, const int32_t *wpos, const int32_t *wneg,
     const long wsz = (long)O * Z, asz = (long)B * Z;
     uint32_t *ws_pos = (uint32_t *)malloc(sizeof(uint32_t) * wsz * T);
     uint32_t *ws_neg = (uint32_t *)malloc(sizeof(uint32_t) * wsz * T);
-    uint32_t *as = (uint32_t *)malloc(sizeof(uint32_t) * asz * T);
+    /* When gen_config does not divide bit_length the activation interleave below reaches slots
+     * past bit_length*gen_config (the reference writes past its buffer there; those slots are
+     * never read).  Size the buffer for the highest slot written so the restatement stays defined. */
+    const int T_act = ((bit_length + g - 1) / g) * g * g;
+    uint32_t *as = (uint32_t *)malloc(sizeof(uint32_t) * asz * (T_act > T ? T_act : T));
     if (!ws_pos || !ws_neg || !as) { free(ws_pos); free(ws_neg); free(as); return -2; }
 
 #pragma omp parallel for schedule(static)

@@ -46,6 +46,7 @@ SIGNATURES = {
     "rexsc_version": (_int, []),
     "rexsc_init": (_int, [_vp]),
     "rexsc_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(ConvDesc)]),
+    "rexsc_conv2d_plan_info": (_int, [ctypes.POINTER(ConvDesc), ctypes.POINTER(ctypes.c_int64)]),
     "rexsc_conv2d_orn": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "rexsc_linear_workspace_bytes": (_sz, [ctypes.POINTER(LinearDesc)]),
     "rexsc_linear_orn": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

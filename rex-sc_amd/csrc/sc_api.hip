@@ -227,6 +227,20 @@ extern "C" size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d)
     return pl.total;
 }
 
+// Planning decisions of the conv op, for tests and tuning: fills out[0..15] with
+// {tuned, KW, ZC, ZG, O_pad, px, ns, splits, slots_per_split, n_slots, direct, n_chunk, M, Hp, Wp, wide}.
+extern "C" int rexsc_conv2d_plan_info(const rexsc_conv_desc *d, int64_t *out)
+{
+    ScPlan pl;
+    int rc = plan_conv(pl, d);
+    if (rc) return rc;
+    const int64_t v[16] = {pl.tuned, pl.KW, pl.ZC, pl.cp.ZG, pl.cp.O_pad, pl.cp.px, pl.cp.ns, pl.cp.splits,
+                           pl.cp.slots_per_split, pl.cp.n_slots, pl.cp.direct, pl.n_chunk, pl.cp.M, pl.cp.Hp,
+                           pl.cp.Wp, pl.wide};
+    for (int i = 0; i < 16; i++) out[i] = v[i];
+    return REXSC_OK;
+}
+
 extern "C" int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
                                 int16_t *out_neg, int16_t *out_diff, void *workspace, size_t workspace_bytes,
                                 rexsc_stream_t stream_)

@@ -188,3 +188,42 @@ def test_quantize_reference_formula():
     assert np.allclose(q * 128, [-127, -128 + 0, -1, 0, 0, 64, 127, 127][:8]) or True
     assert q.max() == 127 / 128 and q.min() == -127 / 128
     assert np.array_equal(orc.quantize(q, 7), q)  # idempotent
+
+
+@pytest.mark.parametrize("g,bc", [(1, 0), (2, 1), (3, 1), (3, -2), (4, 2)])
+def test_linear_slot_interleave_brute_force(g, bc):
+    """The linear op, gen_config g, against a per-bit Python loop: slot s < L pairs activation cycle
+    (s // g^2) * g + s % g with weight cycle s // g (sc_matmul.cpp:422,:667 read only the first L
+    of the L*g generated slots), including g that does not divide L."""
+    L, B, C, O = 8, 2, 37, 3
+    lb, P = 3, 7
+    rng = np.random.default_rng(40 + g)
+    x = (rng.integers(0, L + 1, size=(B, C)) / L).astype(np.float32)
+    w = (rng.integers(-L, L + 1, size=(O, C)) / L).astype(np.float32)
+    xq = np.ceil(np.clip(x * L, 0, L - 1)).astype(int)
+    wp = np.ceil(np.clip(w * L, 0, L - 1)).astype(int)
+    wn = np.ceil(-np.clip(w * L, 1 - L, 0)).astype(int)
+
+    def stream(v, seed):
+        bits, state = [], seed
+        for _ in range(L):
+            state = orc.lfsr_step(lb, 0, state)
+            bits.append(int(v > state))
+        return bits
+
+    a_bits = [[stream(xq[b, c], c % P + 1) for c in range(C)] for b in range(B)]
+    p_bits = [[stream(wp[o, c], (13 + c) % P + 1) for c in range(C)] for o in range(O)]
+    n_bits = [[stream(wn[o, c], (13 + c) % P + 1) for c in range(C)] for o in range(O)]
+    n_sat = bc + 1 if bc >= 0 else 1 - bc
+    exp_p = np.zeros((B, O), np.int32)
+    exp_n = np.zeros((B, O), np.int32)
+    for b in range(B):
+        for o in range(O):
+            for s in range(L):
+                ta, tw = (s // (g * g)) * g + s % g, s // g
+                cp = sum(a_bits[b][c][ta] & p_bits[o][c][tw] for c in range(C))
+                cn = sum(a_bits[b][c][ta] & n_bits[o][c][tw] for c in range(C))
+                exp_p[b, o] += (cp >= n_sat) if bc < 0 else min(cp, n_sat)
+                exp_n[b, o] += (cn >= n_sat) if bc < 0 else min(cn, n_sat)
+    pos, neg = orc.linear_generic_general(x, w, (7, 8, 1), L, -1, bc, g)
+    assert np.array_equal(pos, exp_p) and np.array_equal(neg, exp_n)
