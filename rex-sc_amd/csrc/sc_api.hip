@@ -39,7 +39,8 @@ struct ScPlan {
     int n_chunk;       // images per batch chunk
     int Ho, Wo;
     // workspace (bytes)
-    size_t off_w, off_a, off_part, total;
+    size_t off_w, off_a, off_part, off_tab_a, total;
+    size_t tab_a_words; // state-plane table of the bit-sliced activation generator (0: ballot generator)
 };
 
 int choose_zc(int Z, int KW)
@@ -180,7 +181,9 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     pl.off_w = 0;
     pl.off_a = align_up(w_bytes, WS_ALIGN);
     pl.off_part = pl.off_a + align_up(a_bytes, WS_ALIGN);
-    pl.total = pl.off_part + align_up(part_bytes, WS_ALIGN);
+    pl.off_tab_a = pl.off_part + align_up(part_bytes, WS_ALIGN);
+    pl.tab_a_words = sng_act_table_words(ag, pl.gen_act);
+    pl.total = pl.off_tab_a + align_up(pl.tab_a_words * 4, WS_ALIGN);
     return REXSC_OK;
 }
 
@@ -259,8 +262,9 @@ extern "C" int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const 
     uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
     uint32_t *A = (uint32_t *)(ws + pl.off_a);
     uint32_t *part = (uint32_t *)(ws + pl.off_part);
+    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
 
-    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, stream);
+    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
     if (rc) return rc;
     const size_t in_image = (size_t)d->C * d->H * d->W;
     const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
@@ -270,7 +274,7 @@ extern "C" int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const 
         ComputeParams cp = pl.cp;
         ag.N = nc;
         cp.M = nc * pl.Ho * pl.Wo; // slot stride keeps the full-chunk value: the buffer is laid out for n_chunk images
-        rc = sng_activations(x + n0 * in_image, A, ag, pl.gen_act, stream);
+        rc = sng_activations(x + n0 * in_image, A, tab_a, ag, pl.gen_act, stream);
         if (rc) return rc;
         int16_t *op = out_pos ? out_pos + n0 * out_image : nullptr;
         int16_t *on = out_neg ? out_neg + n0 * out_image : nullptr;
@@ -315,9 +319,10 @@ extern "C" int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, cons
     uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
     uint32_t *A = (uint32_t *)(ws + pl.off_a);
     uint32_t *part = (uint32_t *)(ws + pl.off_part);
-    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, stream);
+    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
+    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
     if (rc) return rc;
-    rc = sng_activations(x, A, pl.ag, pl.gen_act, stream);
+    rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
     if (rc) return rc;
     rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, stream);
     if (rc) return rc;

@@ -23,7 +23,16 @@ struct WeightGeom {
     int ZC, ZG, O_pad;
 };
 
-int sng_activations(const float *x, uint32_t *A, const ActGeom &geo, const GenParams &gp, hipStream_t stream);
-int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, hipStream_t stream);
+// Words of LFSR state-plane table the bit-sliced activation generator needs for this problem, or 0
+// when the ballot generator is the better choice.  geo.N and geo.slot_stride must describe a full batch chunk.
+size_t sng_act_table_words(const ActGeom &geo, const GenParams &gp);
+// table != nullptr selects the bit-sliced generator; the table must have been built by sng_weights()
+// for the same (geo, gp) earlier on the same stream.
+int sng_activations(const float *x, uint32_t *A, const uint32_t *table, const ActGeom &geo, const GenParams &gp,
+                    hipStream_t stream);
+// act_table != nullptr: the launch also builds the activation generator's state-plane table
+// (sng_act_table_words() words) for (*act_geo, *act_gp).
+int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, uint32_t *act_table,
+                const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream);
 
 } // namespace rexsc

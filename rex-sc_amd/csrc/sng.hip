@@ -6,6 +6,8 @@
 //
 // Semantics follow the reference CPU extension: sc_conv.cpp:42-200 (conv), sc_matmul.cpp:3-383
 // (linear); quantisation sc_conv.cpp:316-320.
+#include <stdlib.h>
+#include <string.h>
 #include <utility>
 
 #include "sng.h"
@@ -251,6 +253,332 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
     }
 }
 
+// ---- bit-sliced activation SNG ---------------------------------------------------------------
+// One thread produces one stream word per slot: the 32 channels of word z at padded pixel pp.
+// The 32 quantised values are transposed once into LB bit planes (bit c of plane k = bit k of the
+// value of channel c); the LFSR states of the same 32 channels at every slot come as bit planes
+// from a table that depends only on the geometry (word, slot, pixel index mod seed_mod), and
+// "value > state" for all 32 channels is 2*LB-1 bitwise operations.  Thread i of the grid writes
+// word i of every slot plane, so stores are contiguous and nothing is staged through LDS.
+//
+// Table rows hold one word per pm = (pp * seed_pmul) mod seed_mod: 2^lb words (seed_mod entries and
+// one of padding), or a single word when the seed does not depend on the pixel, as in the linear
+// op.  Lanes of a wave are neighbouring pixels, so one load covers a few cache lines.
+//  * full table T[z][slot][k][pm]: plane k of the states at that slot;
+//  * shift table T[z][tau][pm], tau = cycle + lb - 1: plane 0 only.  A Fibonacci LFSR moves its
+//    bits up by one place per step, so bit k of the state at cycle t is bit 0 of the state at
+//    cycle t - k: consecutive slots share all but one plane, and the kernel slides a window of lb
+//    words along the cycle axis, loading one new word per slot.  Valid when slot == cycle and the
+//    LFSR has no spliced zero state.
+struct ActTableJob {
+    uint32_t *T; // nullptr: nothing to build
+    GenParams gp;
+    int n_words, PM, pitch, seed_cmul;
+    int shift, n_tau;
+};
+
+// Half a wave per table entry (z, slot, pm): lane = channel, one ballot per bit plane.  Waves
+// first_wave, first_wave + n_waves, ... of the caller's grid share the entries; s_seq / s_inv hold
+// the sequence table of job.gp.
+__device__ __forceinline__ void build_state_planes(const ActTableJob &job, const uint8_t *s_seq, const uint8_t *s_inv,
+                                                   unsigned first_wave, unsigned n_waves)
+{
+    const GenParams &gp = job.gp;
+    const int lane = threadIdx.x & 63;
+    const int half = lane >> 5, cc = lane & 31;
+    const int rows = job.shift ? job.n_tau : gp.n_slots; // table rows per word: cycles or slots
+    const unsigned entries = (unsigned)job.n_words * rows * job.PM;
+    const unsigned pairs = (entries + 1) / 2;
+    const int cmul = job.seed_cmul % gp.seed_mod;
+    for (unsigned pair = first_wave; pair < pairs; pair += n_waves) {
+        unsigned e = pair * 2 + half;
+        const bool valid = e < entries;
+        if (!valid) e = entries - 1;
+        const int pm = (int)(e % job.PM);
+        const unsigned sz = e / job.PM;
+        const int s = (int)(sz % rows);
+        const int z = (int)(sz / rows);
+        const int ch = z * 32 + cc;
+        int sd = ((ch % gp.seed_mod) * cmul) % gp.seed_mod + pm;
+        if (sd >= gp.seed_mod) sd -= gp.seed_mod;
+        const int pos = s_inv[sd + 1] + 1;
+        if (job.shift) {
+            int idx = pos + s - (gp.lb - 1); // cycle s - (lb - 1); the sequence has period gp.period
+            if (idx < 0) idx += gp.period;
+            const unsigned long long m = __ballot(s_seq[idx] & 1u);
+            if (valid && cc == 0) job.T[((long)z * rows + s) * job.pitch + pm] = half ? (uint32_t)(m >> 32) : (uint32_t)m;
+            continue;
+        }
+        const uint32_t st = s_seq[pos + slot_cycle(gp, s)];
+        uint32_t mine = 0;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const unsigned long long m = __ballot((st >> k) & 1u);
+            const uint32_t word = half ? (uint32_t)(m >> 32) : (uint32_t)m;
+            if (cc == k) mine = word;
+        }
+        if (valid && cc < gp.lb) job.T[((long)(z * gp.n_slots + s) * gp.lb + cc) * job.pitch + pm] = mine;
+    }
+}
+
+// all 32 channels of one word: value > state, from bit planes (least significant plane first):
+// a higher plane decides wherever it differs, otherwise the result of the lower planes stands
+template <int LB>
+__device__ __forceinline__ uint32_t planes_greater(const uint32_t (&V)[LB], const uint32_t (&S)[LB], int first_plane)
+{
+    uint32_t gt = 0;
+#pragma unroll
+    for (int k = 0; k < LB; k++) {
+        const uint32_t vk = k >= first_plane ? V[k] : 0u; // progressive loading truncates low bits
+        const uint32_t d = vk ^ S[k];
+        gt = (d & vk) | (~d & gt);
+    }
+    return gt;
+}
+
+// One round of the 8x8 bit-matrix transposition between register index and bit position inside
+// every byte: exchanges index bit log2(D) with position bit log2(D).
+template <int D, uint32_t MASK>
+__device__ __forceinline__ void transpose_round(uint32_t &lo, uint32_t &hi)
+{
+    const uint32_t nlo = (lo & MASK) | ((hi << D) & ~MASK);
+    const uint32_t nhi = ((lo >> D) & MASK) | (hi & ~MASK);
+    lo = nlo; hi = nhi;
+}
+
+// 32 quantised values (at most 8 bits each), packed so that byte b of R[j] is the value of channel
+// 8*b + j, become bit planes: afterwards bit c of R[k] is bit k of the value of channel c.
+__device__ __forceinline__ void values_to_planes(uint32_t (&R)[8])
+{
+    transpose_round<1, 0x55555555u>(R[0], R[1]); transpose_round<1, 0x55555555u>(R[2], R[3]);
+    transpose_round<1, 0x55555555u>(R[4], R[5]); transpose_round<1, 0x55555555u>(R[6], R[7]);
+    transpose_round<2, 0x33333333u>(R[0], R[2]); transpose_round<2, 0x33333333u>(R[1], R[3]);
+    transpose_round<2, 0x33333333u>(R[4], R[6]); transpose_round<2, 0x33333333u>(R[5], R[7]);
+    transpose_round<4, 0x0f0f0f0fu>(R[0], R[4]); transpose_round<4, 0x0f0f0f0fu>(R[1], R[5]);
+    transpose_round<4, 0x0f0f0f0fu>(R[2], R[6]); transpose_round<4, 0x0f0f0f0fu>(R[3], R[7]);
+}
+
+// ceil(clamp(v*S, 0, S-1)) of channel c, deposited in its byte of the packed registers
+template <int C>
+__device__ __forceinline__ void pack_quantised(uint32_t (&R)[8], float v, float S)
+{
+    float t = v * S;
+    t = ceilf(fminf(fmaxf(t, 0.f), S - 1.f));
+    R[C & 7] = __builtin_amdgcn_cvt_pk_u8_f32(t, C >> 3, R[C & 7]);
+}
+template <int... C>
+__device__ __forceinline__ void pack_quantised_all(uint32_t (&R)[8], const float (&v)[32], float S,
+                                                   std::integer_sequence<int, C...>)
+{
+    (pack_quantised<C>(R, v[C], S), ...);
+}
+
+template <int LB, bool PIXSEED, bool SHIFT>
+__global__ __launch_bounds__(256) void sng_act_sliced_kernel(const float *__restrict__ x, uint32_t *__restrict__ A,
+                                                             const uint32_t *__restrict__ T, ActGeom geo, GenParams gp,
+                                                             int slots_per_split, int vec4, int log2_zc,
+                                                             int waves_per_plane, int n_waves)
+{
+    // wave-uniform part of the index: which (image, channel chunk) plane, which 64 words of it
+    const int wg = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
+    if (wg >= n_waves) return;
+    const int q = wg / waves_per_plane;
+    const int wb = wg - q * waves_per_plane;
+    const int zg = q % geo.ZG, n = q / geo.ZG;
+    const int HpWp = geo.Hp * geo.Wp;
+    const int plane_words = HpWp << log2_zc;
+    const int rem = wb * 64 + (threadIdx.x & 63);
+    if (rem >= plane_words) return;
+    const int zc = rem & ((1 << log2_zc) - 1);
+    const int pp = rem >> log2_zc;
+    const int z = (zg << log2_zc) + zc;
+    const int c0 = z * 32;
+    const int yp = pp / geo.Wp, xp = pp - yp * geo.Wp;
+    const int y = yp - geo.pad_h, xx = xp - geo.pad_w;
+    const bool inb = y >= 0 && y < geo.H && xx >= 0 && xx < geo.W && c0 < geo.C;
+    const float S = (float)gp.scale;
+
+    uint32_t R[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (inb) {
+        float v[32];
+        if (geo.channels_last) {
+            const float *src = x + (((long)n * geo.H + y) * geo.W + xx) * geo.C + c0;
+            if (vec4 && c0 + 32 <= geo.C) {
+#pragma unroll
+                for (int f4 = 0; f4 < 8; f4++) {
+                    const float4 f = reinterpret_cast<const float4 *>(src)[f4];
+                    v[4 * f4] = f.x; v[4 * f4 + 1] = f.y; v[4 * f4 + 2] = f.z; v[4 * f4 + 3] = f.w;
+                }
+            } else {
+#pragma unroll
+                for (int cc = 0; cc < 32; cc++) v[cc] = c0 + cc < geo.C ? src[cc] : 0.f;
+            }
+        } else {
+            const long plane = (long)geo.H * geo.W;
+            const float *src = x + ((long)n * geo.C + c0) * plane + (long)y * geo.W + xx;
+#pragma unroll
+            for (int cc = 0; cc < 32; cc++) v[cc] = c0 + cc < geo.C ? src[cc * plane] : 0.f;
+        }
+        pack_quantised_all(R, v, S, std::make_integer_sequence<int, 32>{});
+        values_to_planes(R);
+    }
+    uint32_t V[LB];
+#pragma unroll
+    for (int k = 0; k < LB; k++) V[k] = R[k];
+
+    constexpr int PITCH = PIXSEED ? (1 << LB) : 1; // words per table row
+    const int pm = PIXSEED ? ((pp % gp.seed_mod) * (geo.seed_pmul % gp.seed_mod)) % gp.seed_mod : 0;
+    const int s_begin = blockIdx.y * slots_per_split;
+    const int s_end = min(gp.n_slots, s_begin + slots_per_split);
+    uint32_t *dst = A + (long)q * plane_words + rem + (long)s_begin * geo.slot_stride;
+    const int n_mine = s_end - s_begin;
+    // Slots go in groups of U with the table words of the next group requested before the words of
+    // the current one are stored: loads and stores complete in issue order on this hardware, so a
+    // load issued after a store would have to wait for that store as well.
+    constexpr int U = 4;
+    if constexpr (SHIFT) {
+        const int n_tau = gp.n_slots + LB - 1;
+        // row r of T0: plane 0 at cycle s_begin + r - (LB - 1)
+        const uint32_t *T0 = T + ((long)z * n_tau + s_begin) * PITCH + pm;
+        uint32_t W[LB]; // W[k] = plane 0 at cycle (slot - k) = plane k at the current slot
+#pragma unroll
+        for (int k = 0; k < LB; k++) W[k] = T0[(LB - 1 - k) * PITCH];
+        for (int g0 = 0; g0 < n_mine; g0 += U) {
+            uint32_t nxt[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) nxt[u] = T0[(long)(min(g0 + u + 1, n_mine - 1) + LB - 1) * PITCH];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (g0 + u < n_mine) {
+                    const int first = gp.prog ? prog_shift(gp, s_begin + g0 + u) : 0;
+                    dst[(long)(g0 + u) * geo.slot_stride] = planes_greater<LB>(V, W, first);
+                }
+#pragma unroll
+                for (int k = LB - 1; k > 0; k--) W[k] = W[k - 1];
+                W[0] = nxt[u];
+            }
+        }
+    } else {
+        const uint32_t *Ts = T + ((long)z * gp.n_slots + s_begin) * (LB * PITCH) + pm;
+        constexpr int t_step = LB * PITCH;
+        auto load_group = [&](uint32_t (&Sg)[U][LB], int g0) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int su = min(g0 + u, n_mine - 1); // past the end: re-read the last row (unused)
+#pragma unroll
+                for (int k = 0; k < LB; k++) Sg[u][k] = Ts[(long)su * t_step + k * PITCH];
+            }
+        };
+        uint32_t Sa[U][LB];
+        load_group(Sa, 0);
+        for (int g0 = 0; g0 < n_mine; g0 += U) {
+            uint32_t Sb[U][LB];
+            load_group(Sb, g0 + U);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (g0 + u < n_mine) {
+                    const int first = gp.prog ? prog_shift(gp, slot_cycle(gp, s_begin + g0 + u)) : 0;
+                    dst[(long)(g0 + u) * geo.slot_stride] = planes_greater<LB>(V, Sa[u], first);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int k = 0; k < LB; k++) Sa[u][k] = Sb[u][k];
+        }
+    }
+}
+
+// REXSC_SNG_MODE: 0/unset = choose per problem, 1 = always the ballot activation generator,
+// 2 = always the bit-sliced one
+static int sng_mode()
+{
+    const char *e = getenv("REXSC_SNG_MODE");
+    return e ? atoi(e) : 0;
+}
+
+static ActTableJob act_table_job(uint32_t *T, const ActGeom &geo, const GenParams &gp)
+{
+    ActTableJob job;
+    job.T = T;
+    job.gp = gp;
+    job.n_words = geo.ZG * geo.ZC;
+    job.PM = geo.seed_pmul % gp.seed_mod == 0 ? 1 : gp.seed_mod;
+    job.pitch = job.PM == 1 ? 1 : (1 << gp.lb);
+    job.seed_cmul = geo.seed_cmul;
+    job.shift = (!gp.acc && gp.slot_div == 1 && gp.slot_mul == 1 && gp.slot_mod == 1) ? 1 : 0;
+    job.n_tau = gp.n_slots + gp.lb - 1;
+    return job;
+}
+
+static size_t act_table_words_of(const ActTableJob &job)
+{
+    return (size_t)job.n_words * (job.shift ? (size_t)job.n_tau : (size_t)job.gp.n_slots * job.gp.lb) * job.pitch;
+}
+
+size_t sng_act_table_words(const ActGeom &geo, const GenParams &gp)
+{
+    const int mode = sng_mode();
+    if (mode == 1) return 0;
+    const size_t words = act_table_words_of(act_table_job(nullptr, geo, gp));
+    // worth it only when the table is small against the streams it helps to produce
+    if (mode != 2 && words * 8 > (size_t)gp.n_slots * (size_t)geo.slot_stride) return 0;
+    return words;
+}
+
+template <int LB, bool PIXSEED, bool SHIFT>
+static void launch_act_sliced(const float *x, uint32_t *A, const uint32_t *T, const ActGeom &geo, const GenParams &gp,
+                              hipStream_t stream)
+{
+    int log2_zc = 0;
+    while ((1 << log2_zc) < geo.ZC) log2_zc++;
+    const int waves_per_plane = ceil_div(geo.Hp * geo.Wp * geo.ZC, 64);
+    const long n_waves = (long)geo.N * geo.ZG * waves_per_plane;
+    const long blocks = (n_waves + 3) / 4;
+    // few words per slot plane: split the slots over blocks as well (the plane build is repeated)
+    int splits = 1;
+    while (blocks * splits < 2048 && splits * 2 <= gp.n_slots) splits *= 2;
+    const int sps = ceil_div(gp.n_slots, splits);
+    const int vec4 = geo.channels_last && geo.C % 4 == 0 && ((uintptr_t)x % 16 == 0);
+    hipLaunchKernelGGL((sng_act_sliced_kernel<LB, PIXSEED, SHIFT>), dim3((unsigned)blocks, ceil_div(gp.n_slots, sps)),
+                       dim3(256), 0, stream, x, A, T, geo, gp, sps, vec4, log2_zc, waves_per_plane, (int)n_waves);
+}
+
+template <int LB>
+static void launch_act_sliced_lb(const float *x, uint32_t *A, const uint32_t *T, const ActGeom &geo, const GenParams &gp,
+                                 const ActTableJob &job, hipStream_t stream)
+{
+    if (job.PM == 1) {
+        if (job.shift) launch_act_sliced<LB, false, true>(x, A, T, geo, gp, stream);
+        else launch_act_sliced<LB, false, false>(x, A, T, geo, gp, stream);
+    } else {
+        if (job.shift) launch_act_sliced<LB, true, true>(x, A, T, geo, gp, stream);
+        else launch_act_sliced<LB, true, false>(x, A, T, geo, gp, stream);
+    }
+}
+
+// The table must have been built (by the weight generator's launch) for the same geo / gp.
+static int sng_activations_sliced(const float *x, uint32_t *A, const uint32_t *T, const ActGeom &geo, const GenParams &gp,
+                                  hipStream_t stream)
+{
+    const ActTableJob job = act_table_job(nullptr, geo, gp);
+    REXSC_CHECK_ARG((long)geo.N * geo.ZG * ceil_div(geo.Hp * geo.Wp * geo.ZC, 64) < (1L << 31) &&
+                    (geo.ZC & (geo.ZC - 1)) == 0, "activation SNG: problem too large");
+    ProfScope prof("sng_act", 4.0 * geo.N * geo.C * geo.H * geo.W + 4.0 * gp.n_slots * geo.N * geo.ZG * geo.Hp * geo.Wp * geo.ZC,
+                   stream);
+    switch (gp.lb) {
+    case 3: launch_act_sliced_lb<3>(x, A, T, geo, gp, job, stream); break;
+    case 4: launch_act_sliced_lb<4>(x, A, T, geo, gp, job, stream); break;
+    case 5: launch_act_sliced_lb<5>(x, A, T, geo, gp, job, stream); break;
+    case 6: launch_act_sliced_lb<6>(x, A, T, geo, gp, job, stream); break;
+    case 7: launch_act_sliced_lb<7>(x, A, T, geo, gp, job, stream); break;
+    case 8: launch_act_sliced_lb<8>(x, A, T, geo, gp, job, stream); break;
+    default: set_error("activation SNG: unsupported LFSR width %d", gp.lb); return REXSC_ERR_INVALID;
+    }
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
 // ---- weight SNG ------------------------------------------------------------------------------
 // Output layout: Wst[slot][ky][zg][o][pol][kx][zc]  (o padded to O_pad; padded rows are zero).
 // Block: 256 threads, one (group of `wog` output channels, ky, zg); wog is 16, 8, 4 or 2, the largest
@@ -258,71 +586,127 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
 constexpr int W_OG_MAX = 16;
 constexpr int W_SLOT_GROUP = 32; // upper bound; the launcher shrinks it to fit the LDS budget
 
+constexpr int W_COMBO_CHUNK = 8; // (kx, 64-channel half) combinations whose state planes are held in LDS at a time
+
+// Streams of one (kx, 64-channel half, output channel) triple for a group of up to 32 slots:
+//  * lane = channel quantises its weight; one ballot per bit plane and polarity turns the 64 values
+//    into value bit planes that sit in SGPR pairs (low word: channels 0..31, high word: 32..63);
+//  * lane = (word w, slot t) holds the LFSR states of the word's 32 channels at slot t as bit planes
+//    (computed once per block and slot group, shared by all output channels);
+//  * "value > state" for the 32 channels of a word is then 2 bitwise operations per plane, and
+//    the lane ends up with the finished stream word of (slot t, word w), which it puts into the
+//    staging row of slot t.
 template <int ZC>
 __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict__ w, uint32_t *__restrict__ Wst,
                                                          const SeqTable *__restrict__ tables, WeightGeom geo, GenParams gp,
-                                                         int slot_group, int wog)
+                                                         int slot_group, int wog, int n_wblocks, ActTableJob job)
 {
     constexpr int CCH = 32 * ZC;
     constexpr int HALVES = (CCH + 63) / 64;
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     uint8_t *s_seq = s_dyn;
     uint8_t *s_inv = s_dyn + SEQ_LEN;
-    uint32_t *s_stage = reinterpret_cast<uint32_t *>(s_dyn + SEQ_LEN + 256);
+    uint32_t *s_S = reinterpret_cast<uint32_t *>(s_dyn + SEQ_LEN + 256);   // [combo in chunk][plane 0..7][lane]
+    uint32_t *s_stage = s_S + W_COMBO_CHUNK * 8 * 64;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int og = blockIdx.x, ky = blockIdx.y, zg = blockIdx.z;
+    if ((int)blockIdx.x >= n_wblocks) {
+        // extra blocks of the launch build the state-plane table of the activation generator
+        load_tables_to_lds(tables + seq_index(job.gp.lb, job.gp.acc), s_seq, s_inv);
+        __syncthreads();
+        build_state_planes(job, s_seq, s_inv, (blockIdx.x - n_wblocks) * 4 + wave, (gridDim.x - n_wblocks) * 4);
+        return;
+    }
+    const int n_og = geo.O_pad / wog;
+    const int og = blockIdx.x % n_og;
+    const int ky = (blockIdx.x / n_og) % geo.KH;
+    const int zg = blockIdx.x / (n_og * geo.KH);
     const int KW = geo.KW;
     const int row = wog * 2 * KW * ZC; // words per slot handled by this block
     const int pitch = row + 2;          // LDS row pitch (bank spreading for the per-slot writes)
     const float S = (float)gp.scale;
+    const int lb = gp.lb;
+    const int wsel = lane >> 5, t = lane & 31; // this lane's word of the 64-channel half, and slot of the group
+    const int ncombo = KW * HALVES;
+    const int seed_step = (geo.KH * KW) % gp.seed_mod;
 
     load_tables_to_lds(tables + seq_index(gp.lb, gp.acc), s_seq, s_inv);
     __syncthreads();
 
-    const int ntask = wog * KW * HALVES;
-    auto task_weight = [&](int task) -> float {
-        const int h = task % HALVES;
-        const int kx = (task / HALVES) % KW;
-        const int ol = task / (HALVES * KW);
-        const int o = og * wog + ol;
-        const int cl = h * 64 + lane;
-        const int c = zg * CCH + cl;
-        if (task < ntask && cl < CCH && c < geo.C && o < geo.O) {
-            const long wi = geo.channels_last ? (((long)o * geo.KH + ky) * KW + kx) * geo.C + c
-                                              : (((long)o * geo.C + c) * geo.KH + ky) * KW + kx;
-            return w[wi];
-        }
-        return 0.f;
-    };
-
     for (int s0 = 0; s0 < gp.n_slots; s0 += slot_group) {
         const int ns = min(slot_group, gp.n_slots - s0);
-        float f = task_weight(wave);
-        for (int task = wave; task < ntask; task += 4) {
-            const float f_next = task_weight(task + 4); // in flight while this task's slots are generated
-            const int h = task % HALVES;
-            const int kx = (task / HALVES) % KW;
-            const int ol = task / (HALVES * KW);
-            const int cl = h * 64 + lane;
-            const int c = zg * CCH + cl;
-            const int vp = quant_ceil_pos(f, S);
-            const int vn = quant_ceil_neg(f, S);
-            // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
-            const int sd = (int)((13L + (long)c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
-            const int pos = s_inv[sd + 1] + 1;
-            uint32_t plo, phi, nlo, nhi;
-            gen_slots32(s_seq, pos, vp, gp, s0, ns, plo, phi);
-            gen_slots32(s_seq, pos, vn, gp, s0, ns, nlo, nhi);
-            if (lane < ns) {
-                uint32_t *dp = &s_stage[lane * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2];
-                uint32_t *dn = &s_stage[lane * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2];
-                dp[0] = plo; dn[0] = nlo;
-                if (ZC > 1) { dp[1] = phi; dn[1] = nhi; }
+        const int cyc = slot_cycle(gp, s0 + min(t, ns - 1));
+        const int first_plane = gp.prog ? prog_shift(gp, cyc) : 0;
+        for (int combo0 = 0; combo0 < ncombo; combo0 += W_COMBO_CHUNK) {
+            const int ncc = min(W_COMBO_CHUNK, ncombo - combo0);
+            // state planes of this lane's (word, slot) for every combination of the chunk
+            for (int cl = wave; cl < ncc; cl += 4) {
+                const int combo = combo0 + cl;
+                const int h = combo % HALVES, kx = combo / HALVES;
+                const long c_first = (long)zg * CCH + h * 64 + wsel * 32;
+                // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
+                int sd = (int)((13L + c_first * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
+                uint32_t R[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int cc = 0; cc < 32; cc++) {
+                    const int pos = s_inv[sd + 1] + 1;
+                    const uint32_t st = s_seq[pos + cyc];
+                    R[cc & 7] |= st << (8 * (cc >> 3));
+                    sd += seed_step;
+                    if (sd >= gp.seed_mod) sd -= gp.seed_mod;
+                }
+                values_to_planes(R);
+#pragma unroll
+                for (int k = 0; k < 8; k++) s_S[(cl * 8 + k) * 64 + lane] = R[k];
             }
-            f = f_next;
+            __syncthreads();
+
+            const int ntask = wog * ncc;
+            auto task_weight = [&](int task) -> float {
+                const int cl = task % ncc, ol = task / ncc;
+                const int combo = combo0 + cl;
+                const int h = combo % HALVES, kx = combo / HALVES;
+                const int o = og * wog + ol;
+                const int chl = h * 64 + lane;
+                const int c = zg * CCH + chl;
+                if (task < ntask && chl < CCH && c < geo.C && o < geo.O) {
+                    const long wi = geo.channels_last ? (((long)o * geo.KH + ky) * KW + kx) * geo.C + c
+                                                      : (((long)o * geo.C + c) * geo.KH + ky) * KW + kx;
+                    return w[wi];
+                }
+                return 0.f;
+            };
+            float f = task_weight(wave);
+            for (int task = wave; task < ntask; task += 4) {
+                const float f_next = task_weight(task + 4); // in flight while this task's words are generated
+                const int cl = task % ncc, ol = task / ncc;
+                const int combo = combo0 + cl;
+                const int h = combo % HALVES, kx = combo / HALVES;
+                const uint32_t vp = (uint32_t)quant_ceil_pos(f, S);
+                const uint32_t vn = (uint32_t)quant_ceil_neg(f, S);
+                uint32_t gt_p = 0, gt_n = 0;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    if (k < lb) { // wave-uniform
+                        const unsigned long long mp = __ballot((vp >> k) & 1u);
+                        const unsigned long long mn = __ballot((vn >> k) & 1u);
+                        uint32_t vkp = wsel ? (uint32_t)(mp >> 32) : (uint32_t)mp;
+                        uint32_t vkn = wsel ? (uint32_t)(mn >> 32) : (uint32_t)mn;
+                        if (k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
+                        const uint32_t sk = s_S[(cl * 8 + k) * 64 + lane];
+                        const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
+                        gt_p = (dp & vkp) | (~dp & gt_p);
+                        gt_n = (dn & vkn) | (~dn & gt_n);
+                    }
+                }
+                if (t < ns && h * 2 + wsel < ZC) {
+                    s_stage[t * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2 + wsel] = gt_p;
+                    s_stage[t * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2 + wsel] = gt_n;
+                }
+                f = f_next;
+            }
+            __syncthreads();
         }
-        __syncthreads();
         for (int s = 0; s < ns; s++) {
             uint32_t *dst = Wst + ((((long)(s0 + s) * geo.KH + ky) * geo.ZG + zg) * geo.O_pad + og * wog) * 2 * KW * ZC;
             for (int i = tid; i < row; i += 256) dst[i] = s_stage[s * pitch + i];
@@ -344,11 +728,13 @@ static int launch_act(const float *x, uint32_t *A, const SeqTable *tables, const
     return REXSC_OK;
 }
 
-int sng_activations(const float *x, uint32_t *A, const ActGeom &geo, const GenParams &gp, hipStream_t stream)
+int sng_activations(const float *x, uint32_t *A, const uint32_t *table, const ActGeom &geo, const GenParams &gp,
+                    hipStream_t stream)
 {
     const SeqTable *tables = nullptr;
     int rc = get_seq_tables(&tables, stream);
     if (rc) return rc;
+    if (table) return sng_activations_sliced(x, A, table, geo, gp, stream);
     REXSC_CHECK_ARG(geo.ZG <= 65535 && geo.N <= 65535, "activation SNG: grid too large (ZG=%d N=%d)", geo.ZG, geo.N);
     switch (geo.ZC) {
     case 1: return launch_act<1>(x, A, tables, geo, gp, stream);
@@ -361,35 +747,52 @@ int sng_activations(const float *x, uint32_t *A, const ActGeom &geo, const GenPa
 
 template <int ZC>
 static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, const WeightGeom &geo,
-                         const GenParams &gp, hipStream_t stream)
+                         const GenParams &gp, const ActTableJob &job, hipStream_t stream)
 {
     int wog = W_OG_MAX;
     while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < 2048) wog /= 2;
-    dim3 grid(geo.O_pad / wog, geo.KH, geo.ZG);
+    const long n_wblocks = (long)(geo.O_pad / wog) * geo.KH * geo.ZG;
+    // extra blocks for the activation generator's state-plane table: 4 waves x 2 entries per pass
+    long n_tblocks = 0;
+    if (job.T) {
+        const long entries = (long)(act_table_words_of(job) / job.pitch / (job.shift ? 1 : job.gp.lb)) * job.PM;
+        REXSC_CHECK_ARG(entries < (1L << 31), "activation SNG: state table too large");
+        n_tblocks = (entries + 7) / 8;
+        if (n_tblocks > 1024) n_tblocks = 1024;
+    }
+    REXSC_CHECK_ARG(n_wblocks + n_tblocks < (1L << 31), "weight SNG: grid too large");
     const size_t row_bytes = sizeof(uint32_t) * (wog * 2 * geo.KW * ZC + 2);
-    int slot_group = (int)((60 * 1024 - SEQ_LEN - 256) / row_bytes);
+    const size_t fixed = SEQ_LEN + 256 + sizeof(uint32_t) * W_COMBO_CHUNK * 8 * 64;
+    int slot_group = (int)((60 * 1024 - fixed) / row_bytes);
     if (slot_group > W_SLOT_GROUP) slot_group = W_SLOT_GROUP;
     REXSC_CHECK_ARG(slot_group >= 1, "weight SNG: kernel width %d too large for LDS staging", geo.KW);
-    const size_t lds = SEQ_LEN + 256 + row_bytes * slot_group;
+    const size_t lds = fixed + row_bytes * slot_group;
     ProfScope prof("sng_weight", 4.0 * geo.O * geo.C * geo.KH * geo.KW +
                                      4.0 * gp.n_slots * geo.KH * geo.ZG * geo.O_pad * 2 * geo.KW * ZC, stream);
-    hipLaunchKernelGGL(sng_weight_kernel<ZC>, grid, dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group, wog);
+    hipLaunchKernelGGL(sng_weight_kernel<ZC>, dim3((unsigned)(n_wblocks + n_tblocks)), dim3(256), lds, stream, w, Wst, tables,
+                       geo, gp, slot_group, wog, (int)n_wblocks, job);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
 
-int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, hipStream_t stream)
+int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, uint32_t *act_table,
+                const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream)
 {
     const SeqTable *tables = nullptr;
     int rc = get_seq_tables(&tables, stream);
     if (rc) return rc;
     REXSC_CHECK_ARG(geo.O_pad % W_OG_MAX == 0, "weight SNG: O_pad %d not a multiple of %d", geo.O_pad, W_OG_MAX);
-    REXSC_CHECK_ARG(geo.KH <= 65535 && geo.ZG <= 65535, "weight SNG: grid too large");
+    ActTableJob job;
+    memset(&job, 0, sizeof(job));
+    if (act_table) {
+        REXSC_CHECK_ARG(act_geo && act_gp, "weight SNG: activation table requested without its geometry");
+        job = act_table_job(act_table, *act_geo, *act_gp);
+    }
     switch (geo.ZC) {
-    case 1: return launch_weight<1>(w, Wst, tables, geo, gp, stream);
-    case 2: return launch_weight<2>(w, Wst, tables, geo, gp, stream);
-    case 4: return launch_weight<4>(w, Wst, tables, geo, gp, stream);
-    case 8: return launch_weight<8>(w, Wst, tables, geo, gp, stream);
+    case 1: return launch_weight<1>(w, Wst, tables, geo, gp, job, stream);
+    case 2: return launch_weight<2>(w, Wst, tables, geo, gp, job, stream);
+    case 4: return launch_weight<4>(w, Wst, tables, geo, gp, job, stream);
+    case 8: return launch_weight<8>(w, Wst, tables, geo, gp, job, stream);
     default: set_error("weight SNG: unsupported chunk width %d", geo.ZC); return REXSC_ERR_INVALID;
     }
 }

@@ -1,6 +1,8 @@
 """Seeded random configurations of the SC conv / linear ops against the oracle: small shapes with
 awkward sizes (fewer pixels than a wave, channel tails, stream lengths from 2 to 256, both
-generators, both layouts for both operands, strides, asymmetric padding, progressive loading)."""
+generators, both layouts for both operands, strides, asymmetric padding, progressive loading).
+Every configuration runs with both bitstream generators of the library (REXSC_SNG_MODE: 1 = lane
+ballot, 2 = bit-sliced); left alone the library picks one per problem size."""
 import numpy as np
 import pytest
 import torch
@@ -33,12 +35,17 @@ _rng = np.random.default_rng(2024)
 CONV_CFGS = [_rand_conv_cfg(_rng) for _ in range(120)]
 
 
+SNG_MODES = {"ballot": "1", "sliced": "2"}
+
+
+@pytest.mark.parametrize("sng", sorted(SNG_MODES))
 @pytest.mark.parametrize("idx", range(len(CONV_CFGS)))
-def test_conv_fuzz(idx):
+def test_conv_fuzz(idx, sng, monkeypatch):
     import sc_extension_cuda
+    monkeypatch.setenv("REXSC_SNG_MODE", SNG_MODES[sng])
     cfg = CONV_CFGS[idx]
     N, C, H, W, O, KH, KW, s, pad, L, gen, bc, prog, cla, clw = cfg
-    print("conv fuzz", idx, cfg, flush=True)
+    print("conv fuzz", idx, sng, cfg, flush=True)
     rng = np.random.default_rng(1000 + idx)
     dens = min(1.0, 6.0 / (C * KH * KW) + 0.05)
     x = (rng.integers(0, L + 1, size=(N, C, H, W)) / L * (rng.uniform(size=(N, C, H, W)) < 3 * dens)).astype(np.float32)
@@ -74,11 +81,13 @@ def _rand_lin_cfg(rng):
 LIN_CFGS = [_rand_lin_cfg(_rng) for _ in range(60)]
 
 
+@pytest.mark.parametrize("sng", sorted(SNG_MODES))
 @pytest.mark.parametrize("idx", range(len(LIN_CFGS)))
-def test_linear_fuzz(idx):
+def test_linear_fuzz(idx, sng, monkeypatch):
     import sc_extension
+    monkeypatch.setenv("REXSC_SNG_MODE", SNG_MODES[sng])
     B, C, O, L, gen, bc, prog = LIN_CFGS[idx]
-    print("linear fuzz", idx, LIN_CFGS[idx], flush=True)
+    print("linear fuzz", idx, sng, LIN_CFGS[idx], flush=True)
     rng = np.random.default_rng(5000 + idx)
     dens = 1.0 if bc > 100 else min(1.0, 8.0 / C + 0.05)
     x = (rng.integers(0, L + 1, size=(B, C)) / L * (rng.uniform(size=(B, C)) < 2 * dens)).astype(np.float32)
