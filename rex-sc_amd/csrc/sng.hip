@@ -582,7 +582,7 @@ static int sng_activations_sliced(const float *x, uint32_t *A, const uint32_t *T
 // ---- weight SNG ------------------------------------------------------------------------------
 // Output layout: Wst[slot][ky][zg][o][pol][kx][zc]  (o padded to O_pad; padded rows are zero).
 // Block: 256 threads, one (group of `wog` output channels, ky, zg); wog is 16, 8, 4 or 2, the largest
-// that still gives the launch a few thousand blocks.
+// that still gives the launch several hundred blocks.
 constexpr int W_OG_MAX = 16;
 constexpr int W_SLOT_GROUP = 32; // upper bound; the launcher shrinks it to fit the LDS budget
 
@@ -596,39 +596,39 @@ constexpr int W_COMBO_CHUNK = 8; // (kx, 64-channel half) combinations whose sta
 //  * "value > state" for the 32 channels of a word is then 2 bitwise operations per plane, and
 //    the lane ends up with the finished stream word of (slot t, word w), which it puts into the
 //    staging row of slot t.
-template <int ZC>
+template <int ZC, int LB>
 __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict__ w, uint32_t *__restrict__ Wst,
                                                          const SeqTable *__restrict__ tables, WeightGeom geo, GenParams gp,
-                                                         int slot_group, int wog, int n_wblocks, ActTableJob job)
+                                                         int slot_group, int wog, ActTableJob job)
 {
     constexpr int CCH = 32 * ZC;
     constexpr int HALVES = (CCH + 63) / 64;
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     uint8_t *s_seq = s_dyn;
     uint8_t *s_inv = s_dyn + SEQ_LEN;
-    uint32_t *s_S = reinterpret_cast<uint32_t *>(s_dyn + SEQ_LEN + 256);   // [combo in chunk][plane 0..7][lane]
+    uint8_t *s_pos = s_dyn + SEQ_LEN + 256;                                 // [combo in chunk][channel of the half]
+    uint32_t *s_S = reinterpret_cast<uint32_t *>(s_pos + W_COMBO_CHUNK * 64); // [combo in chunk][plane 0..7][lane]
     uint32_t *s_stage = s_S + W_COMBO_CHUNK * 8 * 64;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if ((int)blockIdx.x >= n_wblocks) {
-        // extra blocks of the launch build the state-plane table of the activation generator
-        load_tables_to_lds(tables + seq_index(job.gp.lb, job.gp.acc), s_seq, s_inv);
-        __syncthreads();
-        build_state_planes(job, s_seq, s_inv, (blockIdx.x - n_wblocks) * 4 + wave, (gridDim.x - n_wblocks) * 4);
-        return;
-    }
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wblock = blockIdx.x;
     const int n_og = geo.O_pad / wog;
-    const int og = blockIdx.x % n_og;
-    const int ky = (blockIdx.x / n_og) % geo.KH;
-    const int zg = blockIdx.x / (n_og * geo.KH);
+    const int og = wblock % n_og;
+    const int ky = (wblock / n_og) % geo.KH;
+    const int zg = wblock / (n_og * geo.KH);
     const int KW = geo.KW;
     const int row = wog * 2 * KW * ZC; // words per slot handled by this block
     const int pitch = row + 2;          // LDS row pitch (bank spreading for the per-slot writes)
     const float S = (float)gp.scale;
-    const int lb = gp.lb;
     const int wsel = lane >> 5, t = lane & 31; // this lane's word of the 64-channel half, and slot of the group
     const int ncombo = KW * HALVES;
-    const int seed_step = (geo.KH * KW) % gp.seed_mod;
+    // weight element of (output channel o, channel c, ky, kx): o*o_stride + lane part + h*h_step + kx*kx_mul
+    const long o_stride = (long)geo.C * geo.KH * KW;
+    const long c_lane = (long)zg * CCH + lane;
+    const long lane_off = geo.channels_last ? (long)ky * KW * geo.C + c_lane : (c_lane * geo.KH + ky) * KW;
+    const int h_step = geo.channels_last ? 64 : 64 * geo.KH * KW;
+    const int kx_mul = geo.channels_last ? geo.C : 1;
 
     load_tables_to_lds(tables + seq_index(gp.lb, gp.acc), s_seq, s_inv);
     __syncthreads();
@@ -639,80 +639,97 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
         const int first_plane = gp.prog ? prog_shift(gp, cyc) : 0;
         for (int combo0 = 0; combo0 < ncombo; combo0 += W_COMBO_CHUNK) {
             const int ncc = min(W_COMBO_CHUNK, ncombo - combo0);
+            // cycle position of every channel's seed, lane = channel of the 64-channel half:
+            // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
+            if (s0 == 0 || ncombo > W_COMBO_CHUNK) {
+                for (int cl = wave; cl < ncc; cl += 4) {
+                    const int combo = combo0 + cl;
+                    const int h = combo % HALVES, kx = combo / HALVES;
+                    const long c = (long)zg * CCH + h * 64 + lane;
+                    const int sd = (int)((13L + c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
+                    s_pos[cl * 64 + lane] = s_inv[sd + 1];
+                }
+                __syncthreads();
+            }
             // state planes of this lane's (word, slot) for every combination of the chunk
             for (int cl = wave; cl < ncc; cl += 4) {
-                const int combo = combo0 + cl;
-                const int h = combo % HALVES, kx = combo / HALVES;
-                const long c_first = (long)zg * CCH + h * 64 + wsel * 32;
-                // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
-                int sd = (int)((13L + c_first * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
+                const uint8_t *pos = s_pos + cl * 64 + wsel * 32;
+                const uint8_t *seq = s_seq + 1 + cyc;
                 uint32_t R[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                 for (int cc = 0; cc < 32; cc++) {
-                    const int pos = s_inv[sd + 1] + 1;
-                    const uint32_t st = s_seq[pos + cyc];
+                    const uint32_t st = seq[pos[cc]];
                     R[cc & 7] |= st << (8 * (cc >> 3));
-                    sd += seed_step;
-                    if (sd >= gp.seed_mod) sd -= gp.seed_mod;
                 }
                 values_to_planes(R);
 #pragma unroll
-                for (int k = 0; k < 8; k++) s_S[(cl * 8 + k) * 64 + lane] = R[k];
+                for (int k = 0; k < LB; k++) s_S[(cl * 8 + k) * 64 + lane] = R[k];
             }
             __syncthreads();
 
+            // tasks (output channel ol, combination cl) of this chunk, four apart per wave; all task
+            // bookkeeping is wave-uniform (scalar) arithmetic
             const int ntask = wog * ncc;
-            auto task_weight = [&](int task) -> float {
-                const int cl = task % ncc, ol = task / ncc;
-                const int combo = combo0 + cl;
+            struct Task { int ol, cl; };
+            auto advance = [&](Task &tk) {
+                tk.cl += 4;
+                while (tk.cl >= ncc) { tk.cl -= ncc; tk.ol++; }
+            };
+            auto task_weight = [&](const Task &tk) -> float {
+                const int combo = combo0 + tk.cl;
                 const int h = combo % HALVES, kx = combo / HALVES;
-                const int o = og * wog + ol;
-                const int chl = h * 64 + lane;
-                const int c = zg * CCH + chl;
-                if (task < ntask && chl < CCH && c < geo.C && o < geo.O) {
-                    const long wi = geo.channels_last ? (((long)o * geo.KH + ky) * KW + kx) * geo.C + c
-                                                      : (((long)o * geo.C + c) * geo.KH + ky) * KW + kx;
-                    return w[wi];
-                }
+                const int o = og * wog + tk.ol;
+                // channel of this lane: c = zg*CCH + h*64 + lane, inside the chunk and inside C
+                const int lim = min(geo.C - zg * CCH - h * 64, CCH - h * 64);
+                if (tk.ol < wog && lane < lim && o < geo.O)
+                    return w[(long)o * o_stride + lane_off + (long)h * h_step + kx * kx_mul];
                 return 0.f;
             };
-            float f = task_weight(wave);
+            Task tk = {wave / ncc, wave % ncc}, tk_next = tk;
+            advance(tk_next);
+            float f = task_weight(tk);
             for (int task = wave; task < ntask; task += 4) {
-                const float f_next = task_weight(task + 4); // in flight while this task's words are generated
-                const int cl = task % ncc, ol = task / ncc;
+                const float f_next = task_weight(tk_next); // in flight while this task's words are generated
+                const int cl = tk.cl, ol = tk.ol;
                 const int combo = combo0 + cl;
                 const int h = combo % HALVES, kx = combo / HALVES;
-                const uint32_t vp = (uint32_t)quant_ceil_pos(f, S);
-                const uint32_t vn = (uint32_t)quant_ceil_neg(f, S);
+                // A weight feeds one polarity only (the other one quantises to 0): ballot the planes of
+                // the magnitude ceil(min(|f*S|, S-1)) and split them with the sign mask.  A NaN counts
+                // as negative, as it does in ceil(-clamp(f*S, 1-S, 0)).
+                const uint32_t mag = (uint32_t)(int)ceilf(fminf(fabsf(f * S), S - 1.f));
+                const unsigned long long neg = __ballot(!(f >= 0.f));
                 uint32_t gt_p = 0, gt_n = 0;
 #pragma unroll
-                for (int k = 0; k < 8; k++) {
-                    if (k < lb) { // wave-uniform
-                        const unsigned long long mp = __ballot((vp >> k) & 1u);
-                        const unsigned long long mn = __ballot((vn >> k) & 1u);
-                        uint32_t vkp = wsel ? (uint32_t)(mp >> 32) : (uint32_t)mp;
-                        uint32_t vkn = wsel ? (uint32_t)(mn >> 32) : (uint32_t)mn;
-                        if (k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
-                        const uint32_t sk = s_S[(cl * 8 + k) * 64 + lane];
-                        const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
-                        gt_p = (dp & vkp) | (~dp & gt_p);
-                        gt_n = (dn & vkn) | (~dn & gt_n);
-                    }
+                for (int k = 0; k < LB; k++) {
+                    const unsigned long long m = __ballot((mag >> k) & 1u);
+                    const unsigned long long mp = m & ~neg, mn = m & neg;
+                    uint32_t vkp = wsel ? (uint32_t)(mp >> 32) : (uint32_t)mp;
+                    uint32_t vkn = wsel ? (uint32_t)(mn >> 32) : (uint32_t)mn;
+                    if (k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
+                    const uint32_t sk = s_S[(cl * 8 + k) * 64 + lane];
+                    const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
+                    gt_p = (dp & vkp) | (~dp & gt_p);
+                    gt_n = (dn & vkn) | (~dn & gt_n);
                 }
                 if (t < ns && h * 2 + wsel < ZC) {
                     s_stage[t * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2 + wsel] = gt_p;
                     s_stage[t * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2 + wsel] = gt_n;
                 }
                 f = f_next;
+                tk = tk_next;
+                advance(tk_next);
             }
             __syncthreads();
         }
-        for (int s = 0; s < ns; s++) {
+        for (int s = wave; s < ns; s += 4) {
             uint32_t *dst = Wst + ((((long)(s0 + s) * geo.KH + ky) * geo.ZG + zg) * geo.O_pad + og * wog) * 2 * KW * ZC;
-            for (int i = tid; i < row; i += 256) dst[i] = s_stage[s * pitch + i];
+            for (int i = lane; i < row; i += 64) dst[i] = s_stage[s * pitch + i];
         }
         __syncthreads();
     }
+    // every block also builds its share of the activation generator's state-plane table (same LFSR
+    // width and flavour as the weights, so the sequence table in LDS serves both)
+    if (job.T) build_state_planes(job, s_seq, s_inv, wblock * 4 + wave, gridDim.x * 4);
 }
 
 template <int ZC>
@@ -750,27 +767,37 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
                          const GenParams &gp, const ActTableJob &job, hipStream_t stream)
 {
     int wog = W_OG_MAX;
-    while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < 2048) wog /= 2;
+    // every block computes the state planes of its (ky, zg) once, so blocks should not be too small;
+    // about three per CU keep the chip busy
+    while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < 768) wog /= 2;
     const long n_wblocks = (long)(geo.O_pad / wog) * geo.KH * geo.ZG;
-    // extra blocks for the activation generator's state-plane table: 4 waves x 2 entries per pass
-    long n_tblocks = 0;
+    REXSC_CHECK_ARG(n_wblocks < (1L << 31), "weight SNG: grid too large");
     if (job.T) {
         const long entries = (long)(act_table_words_of(job) / job.pitch / (job.shift ? 1 : job.gp.lb)) * job.PM;
         REXSC_CHECK_ARG(entries < (1L << 31), "activation SNG: state table too large");
-        n_tblocks = (entries + 7) / 8;
-        if (n_tblocks > 1024) n_tblocks = 1024;
+        REXSC_CHECK_ARG(job.gp.lb == gp.lb && job.gp.acc == gp.acc, "activation and weight generators use different LFSRs");
     }
-    REXSC_CHECK_ARG(n_wblocks + n_tblocks < (1L << 31), "weight SNG: grid too large");
     const size_t row_bytes = sizeof(uint32_t) * (wog * 2 * geo.KW * ZC + 2);
-    const size_t fixed = SEQ_LEN + 256 + sizeof(uint32_t) * W_COMBO_CHUNK * 8 * 64;
+    const size_t fixed = SEQ_LEN + 256 + W_COMBO_CHUNK * 64 + sizeof(uint32_t) * W_COMBO_CHUNK * 8 * 64;
     int slot_group = (int)((60 * 1024 - fixed) / row_bytes);
     if (slot_group > W_SLOT_GROUP) slot_group = W_SLOT_GROUP;
     REXSC_CHECK_ARG(slot_group >= 1, "weight SNG: kernel width %d too large for LDS staging", geo.KW);
     const size_t lds = fixed + row_bytes * slot_group;
     ProfScope prof("sng_weight", 4.0 * geo.O * geo.C * geo.KH * geo.KW +
                                      4.0 * gp.n_slots * geo.KH * geo.ZG * geo.O_pad * 2 * geo.KW * ZC, stream);
-    hipLaunchKernelGGL(sng_weight_kernel<ZC>, dim3((unsigned)(n_wblocks + n_tblocks)), dim3(256), lds, stream, w, Wst, tables,
-                       geo, gp, slot_group, wog, (int)n_wblocks, job);
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)n_wblocks), dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group, wog,
+                           job);
+    };
+    switch (gp.lb) {
+    case 3: launch(sng_weight_kernel<ZC, 3>); break;
+    case 4: launch(sng_weight_kernel<ZC, 4>); break;
+    case 5: launch(sng_weight_kernel<ZC, 5>); break;
+    case 6: launch(sng_weight_kernel<ZC, 6>); break;
+    case 7: launch(sng_weight_kernel<ZC, 7>); break;
+    case 8: launch(sng_weight_kernel<ZC, 8>); break;
+    default: set_error("weight SNG: unsupported LFSR width %d", gp.lb); return REXSC_ERR_INVALID;
+    }
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
