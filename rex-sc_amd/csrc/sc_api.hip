@@ -43,6 +43,14 @@ struct ScPlan {
     size_t tab_a_words; // state-plane table of the bit-sliced activation generator (0: ballot generator)
 };
 
+// positive integer tuning knob from the environment
+int tune_env(const char *name, int dflt)
+{
+    const char *e = getenv(name);
+    const int v = e ? atoi(e) : dflt;
+    return v > 0 ? v : dflt;
+}
+
 int choose_zc(int Z, int KW)
 {
     int zc = Z >= 4 ? 4 : (Z >= 2 ? 2 : 1);
@@ -155,14 +163,15 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     // (256 CUs x 4 SIMDs x 3) so that its tail is short; what the tiles and NS do not supply comes
     // from splitting the slots over blocks as well (partials merged by the finalize kernel).
     const int o_tiles = O_pad / OT;
-    cp.px = (!pl.wide && cp.M >= 1024) ? 2 : 1;
+    // REXSC_TUNE_PX_MIN_M (default 1024): fewest output pixels for which a lane takes two of them
+    cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 1024)) ? 2 : 1;
     cp.ns = n_slots >= 8 ? 4 : (n_slots >= 2 ? 2 : 1);
     long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
     int splits = 1;
     const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
     // REXSC_TUNE_ROUNDS (default 4): how many rounds of resident waves a launch should have
     // before slots are split over blocks as well
-    static const int rounds = []() { const char *e = getenv("REXSC_TUNE_ROUNDS"); int v = e ? atoi(e) : 4; return v > 0 ? v : 4; }();
+    const int rounds = tune_env("REXSC_TUNE_ROUNDS", 4);
     if (pl.tuned && waves < (long)rounds * TARGET_WAVES) {
         splits = (int)(((long)rounds * TARGET_WAVES + waves - 1) / waves);
         if (splits > max_splits) splits = max_splits;
