@@ -535,9 +535,12 @@ static void launch_act_sliced(const float *x, uint32_t *A, const uint32_t *T, co
     const int waves_per_plane = ceil_div(geo.Hp * geo.Wp * geo.ZC, 64);
     const long n_waves = (long)geo.N * geo.ZG * waves_per_plane;
     const long blocks = (n_waves + 3) / 4;
-    // few words per slot plane: split the slots over blocks as well (the plane build is repeated)
+    // few words per slot plane: split the slots over blocks as well.  Every split repeats the plane
+    // build, so only launches with less than two blocks per CU are split (REXSC_TUNE_SNG_BLOCKS).
     int splits = 1;
-    while (blocks * splits < 2048 && splits * 2 <= gp.n_slots) splits *= 2;
+    const char *tune = getenv("REXSC_TUNE_SNG_BLOCKS");
+    const long min_blocks = tune && atoi(tune) > 0 ? atoi(tune) : 512;
+    while (blocks * splits < min_blocks && splits * 2 <= gp.n_slots) splits *= 2;
     const int sps = ceil_div(gp.n_slots, splits);
     const int vec4 = geo.channels_last && geo.C % 4 == 0 && ((uintptr_t)x % 16 == 0);
     hipLaunchKernelGGL((sng_act_sliced_kernel<LB, PIXSEED, SHIFT>), dim3((unsigned)blocks, ceil_div(gp.n_slots, sps)),
