@@ -772,7 +772,9 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
     int wog = W_OG_MAX;
     // every block computes the state planes of its (ky, zg) once, so blocks should not be too small;
     // about three per CU keep the chip busy
-    while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < 768) wog /= 2;
+    const char *tune = getenv("REXSC_TUNE_WSNG_BLOCKS");
+    const long min_blocks = tune && atoi(tune) > 0 ? atoi(tune) : 768;
+    while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < min_blocks) wog /= 2;
     const long n_wblocks = (long)(geo.O_pad / wog) * geo.KH * geo.ZG;
     REXSC_CHECK_ARG(n_wblocks < (1L << 31), "weight SNG: grid too large");
     if (job.T) {
