@@ -589,6 +589,8 @@ static int sng_activations_sliced(const float *x, uint32_t *A, const uint32_t *T
 constexpr int W_OG_MAX = 16;
 constexpr int W_SLOT_GROUP = 32; // upper bound; the launcher shrinks it to fit the LDS budget
 
+// s_waitcnt immediate: vmcnt(0), expcnt and lgkmcnt left at their maxima (not waited for)
+constexpr int WAIT_VM0 = 0x0F70;
 constexpr int W_COMBO_CHUNK = 8; // (kx, 64-channel half) combinations whose state planes are held in LDS at a time
 
 // Streams of one (kx, 64-channel half, output channel) triple for a group of up to 32 slots:
@@ -599,7 +601,7 @@ constexpr int W_COMBO_CHUNK = 8; // (kx, 64-channel half) combinations whose sta
 //  * "value > state" for the 32 channels of a word is then 2 bitwise operations per plane, and
 //    the lane ends up with the finished stream word of (slot t, word w), which it puts into the
 //    staging row of slot t.
-template <int ZC, int LB>
+template <int ZC, int LB, bool PROG>
 __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict__ w, uint32_t *__restrict__ Wst,
                                                          const SeqTable *__restrict__ tables, WeightGeom geo, GenParams gp,
                                                          int slot_group, int wog, ActTableJob job)
@@ -639,7 +641,7 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
     for (int s0 = 0; s0 < gp.n_slots; s0 += slot_group) {
         const int ns = min(slot_group, gp.n_slots - s0);
         const int cyc = slot_cycle(gp, s0 + min(t, ns - 1));
-        const int first_plane = gp.prog ? prog_shift(gp, cyc) : 0;
+        const int first_plane = PROG ? prog_shift(gp, cyc) : 0;
         for (int combo0 = 0; combo0 < ncombo; combo0 += W_COMBO_CHUNK) {
             const int ncc = min(W_COMBO_CHUNK, ncombo - combo0);
             // cycle position of every channel's seed, lane = channel of the 64-channel half:
@@ -688,39 +690,53 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
                     return w[(long)o * o_stride + lane_off + (long)h * h_step + kx * kx_mul];
                 return 0.f;
             };
-            Task tk = {wave / ncc, wave % ncc}, tk_next = tk;
-            advance(tk_next);
-            float f = task_weight(tk);
-            for (int task = wave; task < ntask; task += 4) {
-                const float f_next = task_weight(tk_next); // in flight while this task's words are generated
-                const int cl = tk.cl, ol = tk.ol;
-                const int combo = combo0 + cl;
-                const int h = combo % HALVES, kx = combo / HALVES;
-                // A weight feeds one polarity only (the other one quantises to 0): ballot the planes of
-                // the magnitude ceil(min(|f*S|, S-1)) and split them with the sign mask.  A NaN counts
-                // as negative, as it does in ceil(-clamp(f*S, 1-S, 0)).
-                const uint32_t mag = (uint32_t)(int)ceilf(fminf(fabsf(f * S), S - 1.f));
-                const unsigned long long neg = __ballot(!(f >= 0.f));
-                uint32_t gt_p = 0, gt_n = 0;
+            // The weights of Q tasks are requested together, one group ahead of their use.  Loads
+            // complete in issue order, so the wait for the current group is placed before the next
+            // group is requested; a wait after the request would cover the request as well.
+            constexpr int Q = 4;
+            Task cursor = {wave / ncc, wave % ncc};
+            Task tq[Q], tq_next[Q];
+            float cur[Q], nxt[Q];
 #pragma unroll
-                for (int k = 0; k < LB; k++) {
-                    const unsigned long long m = __ballot((mag >> k) & 1u);
-                    const unsigned long long mp = m & ~neg, mn = m & neg;
-                    uint32_t vkp = wsel ? (uint32_t)(mp >> 32) : (uint32_t)mp;
-                    uint32_t vkn = wsel ? (uint32_t)(mn >> 32) : (uint32_t)mn;
-                    if (k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
-                    const uint32_t sk = s_S[(cl * 8 + k) * 64 + lane];
-                    const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
-                    gt_p = (dp & vkp) | (~dp & gt_p);
-                    gt_n = (dn & vkn) | (~dn & gt_n);
+            for (int i = 0; i < Q; i++) { tq[i] = cursor; advance(cursor); cur[i] = task_weight(tq[i]); }
+            for (int base = wave; base < ntask; base += 4 * Q) {
+                __builtin_amdgcn_s_waitcnt(WAIT_VM0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < Q; i++) { tq_next[i] = cursor; advance(cursor); nxt[i] = task_weight(tq_next[i]); }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < Q; i++) {
+                    if (tq[i].ol >= wog) continue; // past the last task (wave-uniform)
+                    const float f = cur[i];
+                    const int cl = tq[i].cl, ol = tq[i].ol;
+                    const int combo = combo0 + cl;
+                    const int h = combo % HALVES, kx = combo / HALVES;
+                    // A weight feeds one polarity only (the other one quantises to 0): ballot the planes
+                    // of the magnitude ceil(min(|f*S|, S-1)) and split them with the sign mask.  A NaN
+                    // counts as negative, as it does in ceil(-clamp(f*S, 1-S, 0)).
+                    const uint32_t mag = (uint32_t)(int)ceilf(fminf(fabsf(f * S), S - 1.f));
+                    const unsigned long long neg = __ballot(!(f >= 0.f));
+                    uint32_t gt_p = 0, gt_n = 0;
+#pragma unroll
+                    for (int k = 0; k < LB; k++) {
+                        const unsigned long long m = __ballot((mag >> k) & 1u);
+                        const unsigned long long mp = m & ~neg, mn = m & neg;
+                        uint32_t vkp = wsel ? (uint32_t)(mp >> 32) : (uint32_t)mp;
+                        uint32_t vkn = wsel ? (uint32_t)(mn >> 32) : (uint32_t)mn;
+                        if (PROG && k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
+                        const uint32_t sk = s_S[(cl * 8 + k) * 64 + lane];
+                        const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
+                        gt_p = (dp & vkp) | (~dp & gt_p);
+                        gt_n = (dn & vkn) | (~dn & gt_n);
+                    }
+                    if (t < ns && h * 2 + wsel < ZC) {
+                        s_stage[t * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2 + wsel] = gt_p;
+                        s_stage[t * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2 + wsel] = gt_n;
+                    }
                 }
-                if (t < ns && h * 2 + wsel < ZC) {
-                    s_stage[t * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2 + wsel] = gt_p;
-                    s_stage[t * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2 + wsel] = gt_n;
-                }
-                f = f_next;
-                tk = tk_next;
-                advance(tk_next);
+#pragma unroll
+                for (int i = 0; i < Q; i++) { cur[i] = nxt[i]; tq[i] = tq_next[i]; }
             }
             __syncthreads();
         }
@@ -795,12 +811,12 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
                            job);
     };
     switch (gp.lb) {
-    case 3: launch(sng_weight_kernel<ZC, 3>); break;
-    case 4: launch(sng_weight_kernel<ZC, 4>); break;
-    case 5: launch(sng_weight_kernel<ZC, 5>); break;
-    case 6: launch(sng_weight_kernel<ZC, 6>); break;
-    case 7: launch(sng_weight_kernel<ZC, 7>); break;
-    case 8: launch(sng_weight_kernel<ZC, 8>); break;
+    case 3: if (gp.prog) launch(sng_weight_kernel<ZC, 3, true>); else launch(sng_weight_kernel<ZC, 3, false>); break;
+    case 4: if (gp.prog) launch(sng_weight_kernel<ZC, 4, true>); else launch(sng_weight_kernel<ZC, 4, false>); break;
+    case 5: if (gp.prog) launch(sng_weight_kernel<ZC, 5, true>); else launch(sng_weight_kernel<ZC, 5, false>); break;
+    case 6: if (gp.prog) launch(sng_weight_kernel<ZC, 6, true>); else launch(sng_weight_kernel<ZC, 6, false>); break;
+    case 7: if (gp.prog) launch(sng_weight_kernel<ZC, 7, true>); else launch(sng_weight_kernel<ZC, 7, false>); break;
+    case 8: if (gp.prog) launch(sng_weight_kernel<ZC, 8, true>); else launch(sng_weight_kernel<ZC, 8, false>); break;
     default: set_error("weight SNG: unsupported LFSR width %d", gp.lb); return REXSC_ERR_INVALID;
     }
     REXSC_CHECK_HIP(hipGetLastError());
