@@ -22,9 +22,9 @@ void set_error(const char *fmt, ...)
 namespace {
 
 constexpr size_t WS_ALIGN = 256;
-// Activation streams of one batch chunk are kept below this many bytes; larger batches are
-// processed chunk by chunk with the weight streams generated once.
-constexpr size_t ACT_STREAM_CAP = (size_t)1 << 30;
+// Activation streams of one batch chunk are kept below this many MiB (REXSC_TUNE_ACT_CAP_MB);
+// larger batches are processed chunk by chunk with the weight streams generated once.
+constexpr int ACT_STREAM_CAP_MB = 1024;
 constexpr int TARGET_WAVES = 3072; // 3 resident waves per SIMD on 256 CUs x 4 SIMDs
 
 struct ScPlan {
@@ -132,8 +132,9 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     const size_t words_per_image_slot = (size_t)ZG * Hp * Wp * ZC;
     const size_t bytes_per_image = words_per_image_slot * n_slots * 4;
     int n_chunk = N;
-    if (bytes_per_image * (size_t)N > ACT_STREAM_CAP) {
-        n_chunk = (int)(ACT_STREAM_CAP / bytes_per_image);
+    const size_t act_cap = (size_t)tune_env("REXSC_TUNE_ACT_CAP_MB", ACT_STREAM_CAP_MB) << 20;
+    if (bytes_per_image * (size_t)N > act_cap) {
+        n_chunk = (int)(act_cap / bytes_per_image);
         if (n_chunk < 1) n_chunk = 1;
     }
     REXSC_CHECK_ARG(words_per_image_slot * n_chunk < ((size_t)1 << 31), "activation plane too large");

@@ -67,6 +67,36 @@ def test_conv_fuzz(idx, sng, monkeypatch):
     assert np.array_equal(neg.cpu().numpy(), oneg)
 
 
+@pytest.mark.parametrize("sng", sorted(SNG_MODES))
+@pytest.mark.parametrize("cla", [False, True])
+def test_conv_batch_chunks(cla, sng, monkeypatch):
+    """Batches whose activation streams exceed the cap are processed in chunks (weight streams and the
+    state table are made once): force a 1 MiB cap and compare with the oracle."""
+    import sc_extension_cuda
+    import _lib
+    import ctypes
+    monkeypatch.setenv("REXSC_SNG_MODE", SNG_MODES[sng])
+    monkeypatch.setenv("REXSC_TUNE_ACT_CAP_MB", "1")
+    N, C, H, W, O, L = 7, 70, 25, 23, 20, 32
+    d = _lib.ConvDesc(N, C, H, W, O, 3, 3, 1, 1, 1, 1, L, -1, 1, 1, 7, 8, 1, int(cla), 0)
+    info = (ctypes.c_int64 * 16)()
+    _lib.check(_lib.lib().rexsc_conv2d_plan_info(ctypes.byref(d), info), "plan_info")
+    assert 1 <= info[11] < N, "the cap should split this batch (n_chunk=%d)" % info[11]
+    print("chunked conv", cla, sng, "n_chunk", info[11], flush=True)
+    rng = np.random.default_rng(77)
+    x = (rng.integers(0, L + 1, size=(N, C, H, W)) / L * (rng.uniform(size=(N, C, H, W)) < 0.2)).astype(np.float32)
+    w = (rng.integers(-L, L + 1, size=(O, C, 3, 3)) / L * (rng.uniform(size=(O, C, 3, 3)) < 0.2)).astype(np.float32)
+    xt = torch.from_numpy(x).cuda()
+    if cla:
+        xt = xt.contiguous(memory_format=torch.channels_last)
+    pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(xt, torch.from_numpy(w).cuda(), L, -1, 16, (1, 1), (1, 1),
+                                                                  (7, 8, 1), 1, 1, True, False)
+    opos, oneg = orc.conv2d_generic_general_split(x, w, L, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1,
+                                                  channels_last_activation=cla)
+    assert np.array_equal(pos.cpu().numpy(), opos)
+    assert np.array_equal(neg.cpu().numpy(), oneg)
+
+
 def _rand_lin_cfg(rng):
     B = int(rng.choice([1, 3, 63, 64, 65, 130, 300]))
     C = int(rng.choice([1, 31, 32, 33, 100, 256, 257, 1000]))
