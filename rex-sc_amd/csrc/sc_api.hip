@@ -167,20 +167,30 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     // REXSC_TUNE_PX_MIN_M (default 1024): fewest output pixels for which a lane takes two of them
     cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 1024)) ? 2 : 1;
     cp.ns = n_slots >= 8 ? 4 : (n_slots >= 2 ? 2 : 1);
-    long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
+    const long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
     int splits = 1;
-    const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
-    // REXSC_TUNE_ROUNDS (default 4): how many rounds of resident waves a launch should have
-    // before slots are split over blocks as well
-    const int rounds = tune_env("REXSC_TUNE_ROUNDS", 4);
-    if (pl.tuned && waves < (long)rounds * TARGET_WAVES) {
-        splits = (int)(((long)rounds * TARGET_WAVES + waves - 1) / waves);
-        if (splits > max_splits) splits = max_splits;
-        if (splits > 8) splits = 8;
+    if (pl.tuned) {
+        // Cost model for splitting the slots over `s` blocks as well: the launch takes
+        // ceil(waves*s / resident waves) rounds of waves, each lasting the wave's share of the work plus
+        // a fixed cost per wave (prologue, LDS reduction, stores).  Powers of two keep the shares even.
+        // REXSC_TUNE_WAVE_OVERHEAD: that fixed cost in VALU instructions; REXSC_TUNE_SPLITS forces s.
+        const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
+        const double work1 = (double)ceil_div(n_slots, cp.ns) * KH * ZG * (4.0 * cp.px * OT * KW * ZC);
+        const double overhead = tune_env("REXSC_TUNE_WAVE_OVERHEAD", 1500);
+        double best = 0;
+        for (int s = 1; s <= max_splits && s <= 8; s *= 2) {
+            const double rounds = (double)((waves * s + TARGET_WAVES - 1) / TARGET_WAVES);
+            const double cost = rounds * (work1 / s + overhead);
+            if (s == 1 || cost < best) { best = cost; splits = s; }
+        }
+        const int forced = tune_env("REXSC_TUNE_SPLITS", 0);
+        if (forced > 0) splits = forced < max_splits ? forced : max_splits;
     }
     cp.slots_per_split = ceil_div(n_slots, splits);
     cp.splits = ceil_div(n_slots, cp.slots_per_split);
     cp.direct = (!linear && cp.splits == 1 && !pl.wide) ? 1 : 0;
+    // partial sums of one split: at most slots_per_split * (largest per-slot count)
+    cp.part_narrow = (!pl.wide && (long)cp.slots_per_split * per_slot_max <= 255) ? 1 : 0;
     if (!pl.tuned) { cp.direct = 1; cp.splits = 1; cp.slots_per_split = n_slots; }
 
     // workspace

@@ -18,6 +18,7 @@ struct ComputeParams {
     uint32_t nn;      // n_sat | n_sat << 16
     int mode;         // 0: min(count, n_sat); 1: count >= n_sat
     int direct;       // 1: the compute kernel writes the int16 outputs itself
+    int part_narrow;  // 1: split partials are stored as uint16 (pos | neg << 8): both sums of a split fit 8 bits
     int out_channels_last;
     int px;           // pixels per lane (1 or 2)
     int ns;           // waves per block; they split the slots of the block among themselves

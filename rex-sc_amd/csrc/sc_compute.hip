@@ -324,7 +324,8 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                 // part[plane][split][m][o] for NHWC; plane 1 only in WIDE mode
                 const long idx = p.out_channels_last ? ((long)split * p.M + m) * p.O_pad + oo
                                                      : ((long)split * p.O_pad + oo) * p.M + m;
-                part[idx] = v;
+                if (!WIDE && p.part_narrow) reinterpret_cast<uint16_t *>(part)[idx] = (uint16_t)((v & 0xffu) | ((v >> 8) & 0xff00u));
+                else part[idx] = v;
                 if (WIDE) part[plane + idx] = vw;
             }
         }
@@ -334,33 +335,50 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
 // Sum the slot-split partials and write the final tensors.
 // conv:   int16 pos / neg / diff, NCHW or NHWC, sums wrap at 16 bits like the reference's.
 // linear: int32 pos / neg [M][O].
-template <bool WIDE, typename OutT>
+// IdxT: unsigned when O*M fits 32 bits (64-bit divisions are slow), unsigned long otherwise.
+template <bool WIDE, typename OutT, typename IdxT>
 __global__ __launch_bounds__(256) void sc_finalize_kernel(const uint32_t *__restrict__ part, ComputeParams p,
                                                           OutT *__restrict__ out_pos, OutT *__restrict__ out_neg,
                                                           OutT *__restrict__ out_diff)
 {
-    const long total = (long)p.O * p.M;
+    const IdxT total = (IdxT)p.O * (IdxT)p.M;
     const long plane = (long)p.splits * p.O_pad * p.M;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long split_stride = (long)p.O_pad * p.M;
+    const uint16_t *part16 = reinterpret_cast<const uint16_t *>(part);
+    for (IdxT i = (IdxT)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (IdxT)gridDim.x * blockDim.x) {
         // i runs in output memory order
-        int o, m;
-        if (p.out_channels_last) { m = (int)(i / p.O); o = (int)(i - (long)m * p.O); }
+        IdxT o, m;
+        if (p.out_channels_last) { m = i / (IdxT)p.O; o = i - m * (IdxT)p.O; }
         else {
-            const long no = i / p.HoWo; // n*O + o
-            const int r = (int)(i - no * p.HoWo), n = (int)(no / p.O);
-            o = (int)(no - (long)n * p.O); m = n * p.HoWo + r;
+            const IdxT no = i / (IdxT)p.HoWo; // n*O + o
+            const IdxT r = i - no * (IdxT)p.HoWo, n = no / (IdxT)p.O;
+            o = no - n * (IdxT)p.O; m = n * (IdxT)p.HoWo + r;
         }
+        const long idx0 = p.out_channels_last ? (long)m * p.O_pad + o : (long)o * p.M + m;
         uint32_t sp = 0, sn = 0;
-        for (int s = 0; s < p.splits; s++) {
-            const long idx = p.out_channels_last ? ((long)s * p.M + m) * p.O_pad + o : ((long)s * p.O_pad + o) * p.M + m;
-            if (WIDE) { sp += part[idx]; sn += part[plane + idx]; }
-            else { const uint32_t v = part[idx]; sp += v & 0xffffu; sn += v >> 16; }
+        // the loads of all splits (at most 8 at a time) are issued before the first sum
+        for (int s0 = 0; s0 < p.splits; s0 += 8) {
+            uint32_t v[8], vw[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                v[u] = 0; vw[u] = 0;
+                if (s0 + u < p.splits) {
+                    const long idx = idx0 + (long)(s0 + u) * split_stride;
+                    if (WIDE) { v[u] = part[idx]; vw[u] = part[plane + idx]; }
+                    else v[u] = p.part_narrow ? (uint32_t)part16[idx] : part[idx];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                if (WIDE) { sp += v[u]; sn += vw[u]; }
+                else if (p.part_narrow) { sp += v[u] & 0xffu; sn += v[u] >> 8; }
+                else { sp += v[u] & 0xffffu; sn += v[u] >> 16; }
+            }
         }
-        const long idx = i;
         const OutT vp = (OutT)sp, vn = (OutT)sn; // int16: wraps
-        if (out_pos) out_pos[idx] = vp;
-        if (out_neg) out_neg[idx] = vn;
-        if (out_diff) out_diff[idx] = (OutT)(vp - vn);
+        if (out_pos) out_pos[i] = vp;
+        if (out_neg) out_neg[i] = vn;
+        if (out_diff) out_diff[i] = (OutT)(vp - vn);
     }
 }
 
@@ -472,9 +490,13 @@ int sc_finalize_i16(const uint32_t *part, const ComputeParams &p, int16_t *out_p
 {
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
-    ProfScope prof("sc_finalize_i16", (double)total * (4.0 * p.splits + 4.0), stream);
-    hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
-                       out_neg, out_diff);
+    ProfScope prof("sc_finalize_i16", (double)total * ((p.part_narrow ? 2.0 : 4.0) * p.splits + 4.0), stream);
+    if (total < (1L << 31))
+        hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
+                           out_neg, out_diff);
+    else
+        hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t, unsigned long>), dim3(grid), dim3(256), 0, stream, part, p,
+                           out_pos, out_neg, out_diff);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
@@ -485,11 +507,12 @@ int sc_finalize_i32(const uint32_t *part, const ComputeParams &p, bool wide, int
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
     ProfScope prof("sc_finalize_i32", (double)total * (4.0 * p.splits * (wide ? 2 : 1) + 8.0), stream);
+    REXSC_CHECK_ARG(total < (1L << 31), "linear: too many outputs (%ld)", total);
     if (wide)
-        hipLaunchKernelGGL((sc_finalize_kernel<true, int32_t>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
+        hipLaunchKernelGGL((sc_finalize_kernel<true, int32_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
                            out_neg, (int32_t *)nullptr);
     else
-        hipLaunchKernelGGL((sc_finalize_kernel<false, int32_t>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
+        hipLaunchKernelGGL((sc_finalize_kernel<false, int32_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
                            out_neg, (int32_t *)nullptr);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
