@@ -9,6 +9,7 @@
 //    clamp fires it keeps firing).  This path works on int8/int16 operands quantised once.
 //  * sequential (add_config >= 1): the OR-style adders are order dependent and are evaluated
 //    product by product in the reference's (c, ky, kx) order.
+#include <stdlib.h>
 #include "profile.h"
 #include "rexsc_common.h"
 
@@ -236,8 +237,11 @@ __global__ void fixed_zero_kernel(int32_t *__restrict__ p, size_t n)
 // and parities) are staged in LDS once per block and read with ds_read_b128, so they cost L2
 // bandwidth once per 256 pixels instead of once per 64.  Per kernel row all KW taps are loaded
 // first, then the 8*KW MFMAs run: one exposed memory latency per row instead of one per tap.
+// PB: 32-pixel blocks per wave.  Two blocks reuse every weight fetch twice; one block makes waves half
+// as long and lighter on registers, which the launcher prefers when the pixel count leaves the
+// last round of 64-pixel waves nearly empty.
 constexpr int FT = 64;
-template <int KW>
+template <int KW, int PB>
 __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restrict__ xq16, const int8_t *__restrict__ wq16,
                                                          const int8_t *__restrict__ wp16, int32_t *__restrict__ out,
                                                          Fixed8Params p)
@@ -247,22 +251,20 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int o_tiles = p.O_pad / FT;
-    const long m_tiles = (p.M + FT - 1) / FT;
-    const long m_groups = (m_tiles + 3) / 4;
+    constexpr int WPX = 32 * PB; // pixels per wave
     long blk = blockIdx.x;
     const int ks = (int)(blk % p.ksplit); blk /= p.ksplit;
     const int otile = (int)(blk % o_tiles);
     const long mtile = (blk / o_tiles) * 4 + wave;   // may be past the end: such a wave only helps staging
-    (void)m_groups;
     const int j = lane & 31, h = lane >> 5;
     const long plane = (long)p.Hp * p.Wp;
     const int taps = p.KH * KW;
 
-    long xoff[2];
-    int mm[2];
+    long xoff[PB];
+    int mm[PB];
 #pragma unroll
-    for (int pb = 0; pb < 2; pb++) {
-        const long m = mtile * FT + pb * 32 + j;
+    for (int pb = 0; pb < PB; pb++) {
+        const long m = mtile * WPX + pb * 32 + j;
         mm[pb] = (int)(m < p.M ? m : p.M - 1);
         const int n = mm[pb] / (p.Ho * p.Wo), r = mm[pb] - n * (p.Ho * p.Wo);
         const int yo = r / p.Wo, xo = r - yo * p.Wo;
@@ -274,11 +276,11 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
     const v4i *wpb = reinterpret_cast<const v4i *>(wp16);
     const long wkk = (long)taps * p.O_pad;
 
-    v16i acc[2][2]; // [channel block][pixel block]
+    v16i acc[2][PB]; // [channel block][pixel block]
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+        for (int b = 0; b < PB; b++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
 
@@ -288,11 +290,13 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
     const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
     // Activation rows are software-pipelined: the KW taps of the next (pair, ky) row are requested
     // before the MFMAs of the current row are issued.
-    v4i b0[KW], b1[KW], n0[KW], n1[KW];
+    v4i bc[PB][KW], bn[PB][KW];
     if (cbp_begin < cbp_end) {
         const v4i *xc = xb + (long)(2 * cbp_begin + h) * plane;
 #pragma unroll
-        for (int kx = 0; kx < KW; kx++) { b0[kx] = xc[xoff[0] + kx]; b1[kx] = xc[xoff[1] + kx]; }
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) bc[pb][kx] = xc[xoff[pb] + kx];
     }
     for (int cbp = cbp_begin; cbp < cbp_end; cbp++) {
         // stage the pair's weights: 2 (h) x taps x 2 (val, par) x 64 (o) 16-byte entries
@@ -312,31 +316,37 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
                 if (cn >= cbp_end) { cn = cbp; kn = ky; }
                 const v4i *xn = xb + (long)(2 * cn + h) * plane + (long)kn * p.Wp;
 #pragma unroll
-                for (int kx = 0; kx < KW; kx++) { n0[kx] = xn[xoff[0] + kx]; n1[kx] = xn[xoff[1] + kx]; }
+                for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                    for (int kx = 0; kx < KW; kx++) bn[pb][kx] = xn[xoff[pb] + kx];
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kx = 0; kx < KW; kx++) {
                 const v4i *wt = sw + (ky * KW + kx) * 2 * FT;
                 const v4i a0 = wt[0], a1 = wt[32], q0 = wt[FT], q1 = wt[FT + 32];
-                const v4i p0 = b0[kx] & ones, p1 = b1[kx] & ones; // activation parities
-                acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b0[kx], acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b1[kx], acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b0[kx], acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b1[kx], acc[1][1], 0, 0, 0);
-                acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, p0, acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, p1, acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, p0, acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, p1, acc[1][1], 0, 0, 0);
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++) {
+                    acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bc[pb][kx], acc[0][pb], 0, 0, 0);
+                    acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bc[pb][kx], acc[1][pb], 0, 0, 0);
+                }
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++) {
+                    const v4i par = bc[pb][kx] & ones; // activation parities
+                    acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, par, acc[0][pb], 0, 0, 0);
+                    acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, par, acc[1][pb], 0, 0, 0);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kx = 0; kx < KW; kx++) { b0[kx] = n0[kx]; b1[kx] = n1[kx]; }
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++) bc[pb][kx] = bn[pb][kx];
         }
     }
     const int HoWo = p.Ho * p.Wo;
 #pragma unroll
-    for (int pb = 0; pb < 2; pb++) {
+    for (int pb = 0; pb < PB; pb++) {
         if (mm[pb] < 0) continue;
         const int n = mm[pb] / HoWo, r0 = mm[pb] - n * HoWo;
 #pragma unroll
@@ -427,9 +437,19 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         q.Hp = p.H + 2 * p.pad_h; q.Wp = p.W + 2 * p.pad_w; q.Ho = p.Ho; q.Wo = p.Wo;
         q.CB = (int)align_up((size_t)ceil_div(p.C, 16), 2); q.M = p.N * p.Ho * p.Wo; q.P2 = p.P2;
         // split the channel-block pairs over waves until the launch has a few thousand of them
-        const long tiles = (long)ceil_div(q.M, FT) * (q.O_pad / FT);
+        int pb = 2;
+        if (getenv("REXSC_TUNE_FIXED_PB")) pb = atoi(getenv("REXSC_TUNE_FIXED_PB")) == 1 ? 1 : 2;
+        const int wpx = 32 * pb;
+        const long tiles = (long)ceil_div(q.M, wpx) * (q.O_pad / FT);
         q.ksplit = 1;
-        while (tiles * q.ksplit < 3072 && q.ksplit * 2 <= q.CB / 2) q.ksplit *= 2;
+        // (the atomic epilogue of a split costs about as much as the MFMA work of a wave: split only
+        // while the launch has fewer wave tiles than about one per SIMD)
+        while (tiles * q.ksplit < 1024 && q.ksplit * 2 <= q.CB / 2) q.ksplit *= 2;
+        if (getenv("REXSC_TUNE_FIXED_KSPLIT")) {
+            q.ksplit = atoi(getenv("REXSC_TUNE_FIXED_KSPLIT"));
+            if (q.ksplit < 1) q.ksplit = 1;
+            if (q.ksplit > q.CB / 2) q.ksplit = q.CB / 2;
+        }
         int8_t *xq16 = (int8_t *)workspace;
         int8_t *wq16 = (int8_t *)workspace + off_w;
         int8_t *wp16 = wq16 + (size_t)q.CB * q.KH * q.KW * q.O_pad * 16;
@@ -446,14 +466,23 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
                 hipLaunchKernelGGL(fixed_zero_kernel, dim3(gridf((long)nout / 4 + 1)), dim3(256), 0, stream, out, nout);
         }
         REXSC_CHECK_HIP(hipGetLastError());
-        const long m_groups = ((long)ceil_div(q.M, FT) + 3) / 4;
+        const long m_groups = ((long)ceil_div(q.M, wpx) + 3) / 4;
         const unsigned grid = (unsigned)(m_groups * (q.O_pad / FT) * q.ksplit);
         const size_t lds = (size_t)2 * q.KH * q.KW * 2 * FT * 16;
         ProfScope prof("fixed_conv_mfma", io_bytes, stream);
         switch (q.KW) {
-        case 1: hipLaunchKernelGGL(fixed_mfma_kernel<1>, dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q); break;
-        case 3: hipLaunchKernelGGL(fixed_mfma_kernel<3>, dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q); break;
-        case 5: hipLaunchKernelGGL(fixed_mfma_kernel<5>, dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q); break;
+        case 1:
+            if (pb == 1) hipLaunchKernelGGL((fixed_mfma_kernel<1, 1>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
+            else hipLaunchKernelGGL((fixed_mfma_kernel<1, 2>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
+            break;
+        case 3:
+            if (pb == 1) hipLaunchKernelGGL((fixed_mfma_kernel<3, 1>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
+            else hipLaunchKernelGGL((fixed_mfma_kernel<3, 2>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
+            break;
+        case 5:
+            if (pb == 1) hipLaunchKernelGGL((fixed_mfma_kernel<5, 1>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
+            else hipLaunchKernelGGL((fixed_mfma_kernel<5, 2>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
+            break;
         default: break; // excluded by fixed_use_mfma
         }
         REXSC_CHECK_HIP(hipGetLastError());
