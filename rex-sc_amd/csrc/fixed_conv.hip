@@ -174,46 +174,47 @@ struct Fixed8Params {
 __global__ __launch_bounds__(256) void fixed_pack_act16_kernel(const float *__restrict__ x, int8_t *__restrict__ xq16,
                                                                Fixed8Params p)
 {
-    // one thread per (n, cb, yp, xp): 16 channels -> 16 bytes
-    const long total = (long)p.N * p.CB * p.Hp * p.Wp;
-    const long stride = (long)gridDim.x * blockDim.x;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int xp = (int)(i % p.Wp);
-        const int yp = (int)((i / p.Wp) % p.Hp);
-        const int cb = (int)((i / ((long)p.Wp * p.Hp)) % p.CB);
-        const int n = (int)(i / ((long)p.Wp * p.Hp * p.CB));
-        const int y = yp - p.pad_h, xx = xp - p.pad_w;
+    // one thread per (n, cb, yp, xp): 16 channels -> 16 bytes.  A block stays inside one (n, cb)
+    // plane (blocks_per_plane blocks each), so the per-thread index arithmetic is one 32-bit division.
+    const unsigned plane = (unsigned)p.Hp * p.Wp;
+    const unsigned blocks_per_plane = (plane + 255) / 256;
+    const unsigned ncb = blockIdx.x / blocks_per_plane, pblk = blockIdx.x - ncb * blocks_per_plane;
+    const unsigned n = ncb / (unsigned)p.CB, cb = ncb - n * (unsigned)p.CB;
+    const long in_plane = (long)p.H * p.W;
+    {
+        const unsigned i = pblk * 256 + threadIdx.x;
+        if (i >= plane) return;
+        const unsigned yp = i / (unsigned)p.Wp, xp = i - yp * (unsigned)p.Wp;
+        const int y = (int)yp - p.pad_h, xx = (int)xp - p.pad_w;
         const bool inb = y >= 0 && y < p.H && xx >= 0 && xx < p.W;
+        const float *src = x + ((long)n * p.C + cb * 16) * in_plane + (long)y * p.W + xx;
         float f[16];
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
-            const int c = cb * 16 + k;
-            f[k] = (inb && c < p.C) ? x[(((long)n * p.C + c) * p.H + y) * p.W + xx] : 0.f;
-        }
+        for (int k = 0; k < 16; k++) f[k] = (inb && (int)(cb * 16 + k) < p.C) ? src[k * in_plane] : 0.f;
         uint32_t wds[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int k = 0; k < 16; k++) wds[k >> 2] |= (uint32_t)(uint8_t)quant_round_pos(f[k], p.P2) << (8 * (k & 3));
-        reinterpret_cast<uint4 *>(xq16)[i] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
+        reinterpret_cast<uint4 *>(xq16)[(long)ncb * plane + i] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
     }
 }
 
 __global__ __launch_bounds__(256) void fixed_pack_w16_kernel(const float *__restrict__ w, int8_t *__restrict__ wq16,
                                                              int8_t *__restrict__ wp16, Fixed8Params p)
 {
-    const long total = (long)p.CB * p.KH * p.KW * p.O_pad;
-    const long stride = (long)gridDim.x * blockDim.x;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const int o = (int)(i % p.O_pad);
-        const int kx = (int)((i / p.O_pad) % p.KW);
-        const int ky = (int)((i / ((long)p.O_pad * p.KW)) % p.KH);
-        const int cb = (int)(i / ((long)p.O_pad * p.KW * p.KH));
+    // one thread per (cb, o, tap), tap fastest: the threads of one (cb, o) read one contiguous run of
+    // the OIHW weights (16 channels x KH*KW taps) between them; each writes its 16-byte entries.
+    const unsigned taps = (unsigned)(p.KH * p.KW);
+    const unsigned total = (unsigned)p.CB * p.O_pad * taps;
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        const unsigned tap = i % taps, co = i / taps;
+        const unsigned o = co % (unsigned)p.O_pad, cb = co / (unsigned)p.O_pad;
         uint32_t vals[4] = {0, 0, 0, 0}, pars[4] = {0, 0, 0, 0};
-        if (o < p.O) {
+        if ((int)o < p.O) {
+            const float *src = w + ((long)o * p.C + cb * 16) * taps + tap;
 #pragma unroll
             for (int k = 0; k < 16; k++) {
-                const int c = cb * 16 + k;
-                if (c < p.C) {
-                    const float f = w[(((long)o * p.C + c) * p.KH + ky) * p.KW + kx];
+                if ((int)(cb * 16 + k) < p.C) {
+                    const float f = src[(long)k * taps];
                     const int q = quant_round_pos(f, p.P2) - quant_round_neg(f, p.P2); // signed
                     const int par = (q & 1) ? (q < 0 ? -1 : 1) : 0;
                     vals[k >> 2] |= (uint32_t)(uint8_t)(int8_t)q << (8 * (k & 3));
@@ -221,8 +222,9 @@ __global__ __launch_bounds__(256) void fixed_pack_w16_kernel(const float *__rest
                 }
             }
         }
-        reinterpret_cast<uint4 *>(wq16)[i] = make_uint4(vals[0], vals[1], vals[2], vals[3]);
-        reinterpret_cast<uint4 *>(wp16)[i] = make_uint4(pars[0], pars[1], pars[2], pars[3]);
+        const long dst = ((long)cb * taps + tap) * p.O_pad + o;
+        reinterpret_cast<uint4 *>(wq16)[dst] = make_uint4(vals[0], vals[1], vals[2], vals[3]);
+        reinterpret_cast<uint4 *>(wp16)[dst] = make_uint4(pars[0], pars[1], pars[2], pars[3]);
     }
 }
 
@@ -458,10 +460,11 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         const double io_bytes = 4.0 * p.N * p.C * p.H * p.W + 4.0 * p.O * p.C * p.KH * p.KW + 4.0 * nout;
         {
             ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 16.0 * q.N * q.CB * q.Hp * q.Wp, stream);
-            hipLaunchKernelGGL(fixed_pack_act16_kernel, dim3(gridf((long)q.N * q.CB * q.Hp * q.Wp)), dim3(256), 0, stream,
-                               x, xq16, q);
-            hipLaunchKernelGGL(fixed_pack_w16_kernel, dim3(gridf((long)q.CB * q.KH * q.KW * q.O_pad)), dim3(256), 0,
-                               stream, w, wq16, wp16, q);
+            const long pack_blocks = (((long)q.Hp * q.Wp + 255) / 256) * q.N * q.CB;
+            REXSC_CHECK_ARG(pack_blocks < (1L << 31) && (long)q.CB * q.O_pad * q.KH * q.KW < (1L << 31), "fixed conv2d: problem too large");
+            hipLaunchKernelGGL(fixed_pack_act16_kernel, dim3((unsigned)pack_blocks), dim3(256), 0, stream, x, xq16, q);
+            hipLaunchKernelGGL(fixed_pack_w16_kernel, dim3(gridf((long)q.CB * q.O_pad * q.KH * q.KW)), dim3(256), 0, stream, w, wq16,
+                               wp16, q);
             if (q.ksplit > 1)
                 hipLaunchKernelGGL(fixed_zero_kernel, dim3(gridf((long)nout / 4 + 1)), dim3(256), 0, stream, out, nout);
         }
