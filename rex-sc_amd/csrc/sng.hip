@@ -1,8 +1,12 @@
 // Stream-number generation (SNG): float operands -> quantised integers -> LFSR bitstreams,
-// packed 32 channels per word.  One wave compares 64 channels against their LFSR states with
-// a single v_cmp; the 64-bit lane mask that lands in an SGPR pair IS two stream words, so no
-// shift/or bit packing is needed.  LFSR states are looked up in a per-width sequence table
-// (any cycle of any seed is one LDS byte read), so slots can be produced in any order.
+// packed 32 channels per word.  LFSR states are looked up in a per-width sequence table (any cycle
+// of any seed is one byte read), so slots can be produced in any order.  Three generators:
+//  * sng_act_sliced_kernel: one thread per stream word, bit-plane ("bit-sliced") comparison of 32
+//    channels at once against state planes from a small geometry-only table;
+//  * sng_act_kernel: lane = channel, one v_cmp per slot whose 64-bit lane mask IS two stream
+//    words (for problems too small to amortise the table);
+//  * sng_weight_kernel: ballots for the weight bit planes, bit-sliced comparison per (word, slot)
+//    lane, rows staged in LDS in the order the compute kernel reads them.
 //
 // Semantics follow the reference CPU extension: sc_conv.cpp:42-200 (conv), sc_matmul.cpp:3-383
 // (linear); quantisation sc_conv.cpp:316-320.
@@ -60,13 +64,6 @@ __device__ __forceinline__ int quant_ceil_pos(float v, float S)
     t = fminf(fmaxf(t, 0.f), S - 1.f);
     return (int)ceilf(t);
 }
-__device__ __forceinline__ int quant_ceil_neg(float v, float S)
-{   // ceil(-clamp(v*S, 1-S, 0))
-    float t = v * S;
-    t = fminf(fmaxf(t, 1.f - S), 0.f);
-    return (int)ceilf(-t);
-}
-
 __device__ __forceinline__ void load_tables_to_lds(const SeqTable *tab, uint8_t *seq, uint8_t *inv)
 {
     const uint32_t *src = reinterpret_cast<const uint32_t *>(tab->seq);
