@@ -15,8 +15,9 @@ The one JSON line printed at the end also carries
   roofline      the dominant kernel (AND/popcount compute) against the VALU integer peak:
                 achieved = algorithmic lane-ops / duration measured with HIP events on the launch
                 stream, peak = 256 CU x 64 lanes/clk x 2.4 GHz;
-  cpu_baseline  the C restatement of the reference CPU extension (oracle/, OpenMP) on a bounded
-                sample of the same workload, timed on this host;
+  cpu_baseline  the reference's own CPU extension (compiled into oracle/_ref/) on a bounded sample
+                of the same workload, timed on this host; the C restatement in oracle/ (OpenMP)
+                beside it, and instead of it where the reference build is absent;
   extra         the other reference configurations (SC conv OR-1, SC linear fwd+bwd, fixed-point
                 conv, pointwise kernels, training steps), each with its own rate.
 """
@@ -169,9 +170,32 @@ def main():
     return 0
 
 
+_REF_CHILD = r"""
+import json, sys, time
+sys.path.insert(0, sys.argv[1])
+import numpy as np, torch
+import sc_extension
+layers = json.loads(sys.argv[2]); batch = int(sys.argv[3]); L = int(sys.argv[4]); or_n = int(sys.argv[5])
+rng = np.random.default_rng(5)
+ops = []
+for (C, H, O, K, s) in layers:
+    x = torch.from_numpy((rng.integers(0, L, size=(batch, C, H, H)) / L).astype(np.float32))
+    w = torch.from_numpy((rng.integers(-L + 1, L, size=(O, C, K, K)) / L).astype(np.float32))
+    ops.append((x.contiguous(memory_format=torch.channels_last), w, K, s))
+t0 = time.perf_counter()
+for (x, w, K, s) in ops:
+    sc_extension.conv2d_generic_general(x, w, L, -1, 16, (K // 2, K // 2), (s, s), (7, 8, 1), or_n - 1, 1, True, False)
+print(json.dumps({"sec": time.perf_counter() - t0, "threads": torch.get_num_threads()}))
+"""
+
+
 def cpu_baseline(sample_batch, L, or_n):
-    """The oracle (C restatement of the reference CPU extension, OpenMP) on the same 19 layers at a
-    reduced batch; bit-MAC/s scales linearly with batch for this embarrassingly parallel op."""
+    """CPU rate of the same 19 layers on this host, on a bounded sample (bit-MAC/s scales linearly
+    with batch for this embarrassingly parallel op).  Preferred: the reference's own CPU extension,
+    compiled from its sources into oracle/_ref/ (kind "reference"), run in a child process so that a
+    missing build or an instruction this host lacks cannot take the benchmark down.  Otherwise the C
+    restatement in oracle/ (kind "port"), which is also timed and reported as port_value."""
+    import subprocess
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import numpy as np
     import oracle as orc
@@ -186,9 +210,26 @@ def cpu_baseline(sample_batch, L, or_n):
                                          channels_last_activation=True)
         mac += layer_macs(sample_batch, C, H, O, K, s)
     sec = time.perf_counter() - t0
-    return {"value": mac * L / sec, "unit": "bit-MAC/s", "cores": cores, "kind": "port",
+    port = {"value": mac * L / sec, "unit": "bit-MAC/s", "cores": cores, "kind": "port",
             "sample": "same 19 ResNet-18 SC conv layers at batch %d (%.1f s of CPU time on %d threads)"
                       % (sample_batch, sec, cores)}
+    ref_dir = os.path.join(ROOT, "oracle", "_ref")
+    ref_batch = max(1, sample_batch // 4)
+    if not os.path.exists(os.path.join(ref_dir, "sc_extension.so")):
+        port["reference_skipped"] = "oracle/_ref/sc_extension.so not built"
+        return port
+    try:
+        out = subprocess.run([sys.executable, "-c", _REF_CHILD, ref_dir, json.dumps(RESNET18_SC_LAYERS), str(ref_batch),
+                              str(L), str(or_n)], capture_output=True, text=True, timeout=180)
+        res = json.loads(out.stdout.strip().splitlines()[-1])
+        rmac = sum(layer_macs(ref_batch, C, H, O, K, s) for (C, H, O, K, s) in RESNET18_SC_LAYERS)
+        return {"value": rmac * L / res["sec"], "unit": "bit-MAC/s", "cores": res["threads"], "kind": "reference",
+                "sample": "same 19 ResNet-18 SC conv layers at batch %d through the reference's compiled CPU extension "
+                          "(%.1f s on %d threads)" % (ref_batch, res["sec"], res["threads"]),
+                "port_value": port["value"], "port_sample": port["sample"]}
+    except Exception as e:  # missing build, illegal instruction, timeout: report the port
+        port["reference_skipped"] = "%s: %s" % (type(e).__name__, str(e)[:200])
+        return port
 
 
 if __name__ == "__main__":
