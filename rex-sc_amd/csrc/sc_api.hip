@@ -180,7 +180,14 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
         double best = 0;
         for (int s = 1; s <= max_splits && s <= 8; s *= 2) {
             const double rounds = (double)((waves * s + TARGET_WAVES - 1) / TARGET_WAVES);
-            const double cost = rounds * (work1 / s + overhead);
+            double cost = rounds * (work1 / s + overhead);
+            if (s > 1) {
+                // the finalize pass: launch (~8 us) + partial and output bytes at ~3 TB/s, converted to the
+                // model's unit (one VALU instruction of a wave sharing its SIMD with two others ~ 5.1 ns)
+                const bool narrow = (long)ceil_div(n_slots, s) * per_slot_max <= 255;
+                const double bytes = (double)cp.M * O_pad * ((narrow ? 2.0 : 4.0) * s + 4.0);
+                cost += (8e3 + bytes / 3e3) / 5.1;
+            }
             if (s == 1 || cost < best) { best = cost; splits = s; }
         }
         const int forced = tune_env("REXSC_TUNE_SPLITS", 0);
