@@ -23,6 +23,7 @@ struct ComputeParams {
     int px;           // pixels per lane (1 or 2)
     int ns;           // waves per block; they split the slots of the block among themselves
     int m_tiles, o_tiles; // filled by the launcher
+    int vec_out;          // filled by the launcher: channels-last results may leave as 8-byte stores
 };
 
 int sc_compute_tile_ot();

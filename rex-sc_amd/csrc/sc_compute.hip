@@ -282,7 +282,7 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
         slot = slot_n; ky = ky_n; zg = zg_n;
     }
 
-    // epilogue: sum the NS partial tiles in LDS; each wave then finishes every ns-th accumulator
+    // epilogue: sum the NS partial tiles in LDS
     if (ns > 1) {
 #pragma unroll
         for (int px = 0; px < PX; px++)
@@ -293,40 +293,77 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
             }
         __syncthreads();
     }
+    // Each wave finishes a contiguous group of OT/ns output channels, four at a time: in channels-last
+    // order the four values of a lane are adjacent in memory and leave as one 8- or 16-byte store.
     const long plane = (long)p.splits * p.O_pad * p.M;
+    const int group = OT / ns; // output channels per wave: 16, 8 or 4
 #pragma unroll
     for (int px = 0; px < PX; px++) {
         const int m = mpix[px];
         const int n = m / p.HoWo, r = m - n * p.HoWo;
 #pragma unroll
-        for (int o = 0; o < OT; o++) {
-            if (((px * OT + o) % ns) != wave) continue; // wave-uniform
-            uint32_t v = acc[px][o], vw = WIDE ? accw[px][o] : 0;
-            if (ns > 1) {
-                v = 0; vw = 0;
-                for (int w = 0; w < ns; w++) {
-                    if (WIDE) { v += s_red[w][0][px * OT + o][lane]; vw += s_red[w][1][px * OT + o][lane]; }
-                    else v = pk_add_u16(v, s_red[w][0][px * OT + o][lane]);
+        for (int q = 0; q < OT / 4; q++) {
+            if ((q * 4) / group != wave) continue; // wave-uniform
+            uint32_t v[4], vw[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int o = q * 4 + e;
+                v[e] = acc[px][o]; vw[e] = WIDE ? accw[px][o] : 0;
+                if (ns > 1) {
+                    v[e] = 0; vw[e] = 0;
+                    for (int w = 0; w < ns; w++) {
+                        if (WIDE) { v[e] += s_red[w][0][px * OT + o][lane]; vw[e] += s_red[w][1][px * OT + o][lane]; }
+                        else v[e] = pk_add_u16(v[e], s_red[w][0][px * OT + o][lane]);
+                    }
                 }
             }
             if (m >= p.M) continue;
-            const int oo = otile * OT + o;
+            const int oo = otile * OT + q * 4;
             if (p.direct) {
-                if (oo >= p.O) continue;
-                const long idx = p.out_channels_last ? (long)m * p.O + oo : ((long)n * p.O + oo) * p.HoWo + r;
-                const int16_t vp = (int16_t)(v & 0xffffu), vn = (int16_t)(v >> 16);
-                if (out_pos) out_pos[idx] = vp;
-                if (out_neg) out_neg[idx] = vn;
-                if (out_diff) out_diff[idx] = (int16_t)(vp - vn);
-            } else {
+                if (p.out_channels_last && p.vec_out && oo + 3 < p.O) {
+                    const long idx = (long)m * p.O + oo;
+                    const uint2 vp = make_uint2((v[0] & 0xffffu) | (v[1] << 16), (v[2] & 0xffffu) | (v[3] << 16));
+                    const uint2 vn = make_uint2((v[0] >> 16) | (v[1] & 0xffff0000u), (v[2] >> 16) | (v[3] & 0xffff0000u));
+                    if (out_pos) *reinterpret_cast<uint2 *>(out_pos + idx) = vp;
+                    if (out_neg) *reinterpret_cast<uint2 *>(out_neg + idx) = vn;
+                    if (out_diff) {
+                        const uint32_t d0 = (v[0] - (v[0] >> 16)) & 0xffffu, d1 = (v[1] - (v[1] >> 16)) & 0xffffu;
+                        const uint32_t d2 = (v[2] - (v[2] >> 16)) & 0xffffu, d3 = (v[3] - (v[3] >> 16)) & 0xffffu;
+                        *reinterpret_cast<uint2 *>(out_diff + idx) = make_uint2(d0 | (d1 << 16), d2 | (d3 << 16));
+                    }
+                    continue;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    if (oo + e >= p.O) continue;
+                    const long idx = p.out_channels_last ? (long)m * p.O + oo + e : ((long)n * p.O + oo + e) * p.HoWo + r;
+                    const int16_t vp = (int16_t)(v[e] & 0xffffu), vn = (int16_t)(v[e] >> 16);
+                    if (out_pos) out_pos[idx] = vp;
+                    if (out_neg) out_neg[idx] = vn;
+                    if (out_diff) out_diff[idx] = (int16_t)(vp - vn);
+                }
+            } else if (p.out_channels_last) {
                 // partial sums of a global slot split, laid out like the final tensor so that the
-                // finalize pass is coalesced on both sides: part[plane][split][o][m] for NCHW,
-                // part[plane][split][m][o] for NHWC; plane 1 only in WIDE mode
-                const long idx = p.out_channels_last ? ((long)split * p.M + m) * p.O_pad + oo
-                                                     : ((long)split * p.O_pad + oo) * p.M + m;
-                if (!WIDE && p.part_narrow) reinterpret_cast<uint16_t *>(part)[idx] = (uint16_t)((v & 0xffu) | ((v >> 8) & 0xff00u));
-                else part[idx] = v;
-                if (WIDE) part[plane + idx] = vw;
+                // finalize pass is coalesced on both sides: part[plane][split][m][o] for NHWC,
+                // part[plane][split][o][m] for NCHW; plane 1 only in WIDE mode
+                const long idx = ((long)split * p.M + m) * p.O_pad + oo; // multiple of 4
+                if (!WIDE && p.part_narrow) {
+                    uint32_t h[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) h[e] = (v[e] & 0xffu) | ((v[e] >> 8) & 0xff00u);
+                    *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(part) + idx) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
+                } else {
+                    *reinterpret_cast<uint4 *>(part + idx) = make_uint4(v[0], v[1], v[2], v[3]);
+                    if (WIDE) *reinterpret_cast<uint4 *>(part + plane + idx) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const long idx = ((long)split * p.O_pad + oo + e) * p.M + m;
+                    if (!WIDE && p.part_narrow) reinterpret_cast<uint16_t *>(part)[idx] = (uint16_t)((v[e] & 0xffu) | ((v[e] >> 8) & 0xff00u));
+                    else part[idx] = v[e];
+                    if (WIDE) part[plane + idx] = vw[e];
+                }
             }
         }
     }
@@ -426,6 +463,9 @@ static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams 
 {
     p.m_tiles = ceil_div(p.M, 64 * PX);
     p.o_tiles = p.O_pad / OT;
+    // 8-byte stores of four adjacent int16 results need O % 4 == 0 and 8-byte aligned tensors
+    p.vec_out = (p.O % 4 == 0 && ((uintptr_t)out_pos % 8) == 0 && ((uintptr_t)out_neg % 8) == 0 &&
+                 ((uintptr_t)out_diff % 8) == 0) ? 1 : 0;
     REXSC_CHECK_ARG(p.ns >= 1 && p.ns <= MAX_NS, "SC compute: %d waves per block not supported", p.ns);
     const long blocks = (long)p.m_tiles * p.o_tiles * p.splits;
     REXSC_CHECK_ARG(blocks < (1L << 30), "SC compute: grid too large (%ld blocks)", blocks);
