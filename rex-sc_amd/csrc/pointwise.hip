@@ -283,6 +283,8 @@ __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_backward_kernel(const
 constexpr int CAL_MAX_WIN = 64;
 struct CalWindows { float lo[CAL_MAX_WIN]; float hi[CAL_MAX_WIN]; };
 
+constexpr int CAL_E = 16; // elements a thread holds in registers while it walks the windows
+
 __global__ __launch_bounds__(256) void calib_stats_kernel(const float *__restrict__ a_bit,
                                                           const float *__restrict__ a_act, size_t n, CalWindows w,
                                                           int n_win, double *__restrict__ stats)
@@ -290,20 +292,32 @@ __global__ __launch_bounds__(256) void calib_stats_kernel(const float *__restric
     __shared__ double s_acc[CAL_MAX_WIN * 3];
     for (int i = threadIdx.x; i < n_win * 3; i += blockDim.x) s_acc[i] = 0.0;
     __syncthreads();
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    // Each thread keeps the sums of ONE window at a time in registers: loop windows outermost
-    // over a thread-private slice would re-read memory, so instead accumulate per element into
-    // LDS with wave-level pre-reduction.
-    for (size_t i0 = (size_t)blockIdx.x * blockDim.x; i0 < n; i0 += stride) {
-        const size_t i = i0 + threadIdx.x;
-        const bool ok = i < n;
-        const float act = ok ? a_act[i] : 0.f;
-        const float err = ok ? a_bit[i] - act : 0.f;
+    // A thread loads CAL_E elements (coalesced across the block), then walks the windows with the
+    // elements in registers: per window a few VALU operations per element, one wave reduction and
+    // three LDS atomics per wave.  Partial sums of at most 64*CAL_E terms are kept in float, the
+    // running totals in double.
+    const size_t tile = (size_t)blockDim.x * CAL_E;
+    for (size_t t0 = (size_t)blockIdx.x * tile; t0 < n; t0 += (size_t)gridDim.x * tile) {
+        float act[CAL_E], err[CAL_E];
+#pragma unroll
+        for (int j = 0; j < CAL_E; j++) {
+            const size_t i = t0 + (size_t)j * blockDim.x + threadIdx.x;
+            const bool ok = i < n;
+            act[j] = ok ? a_act[i] : __builtin_nanf(""); // NaN belongs to no window
+            err[j] = ok ? a_bit[i] - act[j] : 0.f;
+        }
         for (int k = 0; k < n_win; k++) {
-            const bool in = ok && act >= w.lo[k] && act < w.hi[k];
-            const unsigned long long m = __ballot(in);
-            if (m == 0) continue; // wave-uniform
-            double c = in ? 1.0 : 0.0, e = in ? (double)err : 0.0, e2 = in ? (double)err * (double)err : 0.0;
+            const float lo = w.lo[k], hi = w.hi[k];
+            float c = 0.f, e = 0.f, e2 = 0.f;
+#pragma unroll
+            for (int j = 0; j < CAL_E; j++) {
+                const bool in = act[j] >= lo && act[j] < hi;
+                const float x = in ? err[j] : 0.f;
+                c += in ? 1.f : 0.f;
+                e += x;
+                e2 = fmaf(x, x, e2);
+            }
+            if (__ballot(c > 0.f) == 0) continue; // wave-uniform
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) {
                 c += __shfl_down(c, off);
@@ -311,9 +325,9 @@ __global__ __launch_bounds__(256) void calib_stats_kernel(const float *__restric
                 e2 += __shfl_down(e2, off);
             }
             if ((threadIdx.x & 63) == 0) {
-                atomicAdd(&s_acc[k * 3 + 0], c);
-                atomicAdd(&s_acc[k * 3 + 1], e);
-                atomicAdd(&s_acc[k * 3 + 2], e2);
+                atomicAdd(&s_acc[k * 3 + 0], (double)c);
+                atomicAdd(&s_acc[k * 3 + 1], (double)e);
+                atomicAdd(&s_acc[k * 3 + 2], (double)e2);
             }
         }
     }
@@ -459,7 +473,8 @@ extern "C" int rexsc_calib_stats(const float *a_bit, const float *a_act, size_t 
     hipLaunchKernelGGL(zero_f64_kernel, dim3(1), dim3(256), 0, stream, stats, n_win * 3);
     REXSC_CHECK_HIP(hipGetLastError());
     if (n == 0) return REXSC_OK;
-    const int grid = pw_grid(n);
+    size_t tiles = (n + 256 * CAL_E - 1) / (256 * CAL_E);
+    const int grid = (int)(tiles < 4096 ? tiles : 4096);
     ProfScope prof("calib_stats", 8.0 * n, stream);
     hipLaunchKernelGGL(calib_stats_kernel, dim3(grid), dim3(256), 0, stream, a_bit, a_act, n, w, n_win, stats);
     REXSC_CHECK_HIP(hipGetLastError());

@@ -148,5 +148,7 @@ def test_calib_stats_kernel():
         sel = (a_act >= lo[k]) & (a_act < hi[k])
         err = (a_bit[sel] - a_act[sel]).astype(np.float64)
         assert st[k, 0] == sel.sum()
-        assert np.isclose(st[k, 1], err.sum(), rtol=1e-9, atol=1e-9)
-        assert np.isclose(st[k, 2], (err * err).sum(), rtol=1e-9, atol=1e-9)
+        # partial sums of up to 1024 terms are float32, the totals float64 (the reference works in
+        # float32 throughout): 1e-6 of the sum of magnitudes
+        assert abs(st[k, 1] - err.sum()) <= 1e-6 * np.abs(err).sum() + 1e-9
+        assert np.isclose(st[k, 2], (err * err).sum(), rtol=1e-6, atol=1e-9)
