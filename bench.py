@@ -137,9 +137,9 @@ def main():
         "achieved": achieved / 1e12, "peak": VALU_PEAK_LANEOPS / 1e12, "unit": "Tlane-op/s",
         "frac": achieved / VALU_PEAK_LANEOPS,
         # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the stage-2
-        # 3x3 layer (profiles/sc_compute_3x3_c128_hbm_traffic.md): 48.9 MB read + 25.7 MB written
+        # 3x3 layer (profiles/sc_compute_3x3_c128_hbm_traffic.md): 39.5 MB read + 25.7 MB written
         # against 56.4 MB algorithmic; at these rates the kernel is nowhere near the HBM roof.
-        "traffic": 74.6e6, "traffic_shape": "128->128 3x3 28x28 batch 64",
+        "traffic": 65.2e6, "traffic_shape": "128->128 3x3 28x28 batch 64",
         "avg_launch_us": dom["total_ms"] * 1e3 / dom["calls"], "launches": dom["calls"],
         "all_compute_kernels_frac": comp_ops / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS,
         "whole_step_frac": (total_mac * L * 4 / 32) / sec / VALU_PEAK_LANEOPS,
