@@ -82,7 +82,9 @@ __device__ __forceinline__ void and_popc_acc(uint32_t &count, uint32_t a, uint32
 
 // One weight batch: G output channels starting at o0, both polarities, all KWZ words, PX pixels.
 // wb holds [g][pol][j].
-template <int PX, int OT, int KWZ, int G>
+// OR1: the slot result is min(count, 1), i.e. "any product bit set": the AND results are OR-ed into
+// the counter registers (one v_and_or_b32 per word) instead of being counted.
+template <int PX, int OT, int KWZ, int G, bool OR1>
 __device__ __forceinline__ void compute_batch(const uint32_t (&a)[PX][KWZ], const uint32_t (&wb)[G * 2 * KWZ],
                                               uint32_t (&cp)[PX][OT], uint32_t (&cn)[PX][OT], int o0)
 {
@@ -94,8 +96,13 @@ __device__ __forceinline__ void compute_batch(const uint32_t (&a)[PX][KWZ], cons
             const uint32_t wn = wb[(g * 2 + 1) * KWZ + j];
 #pragma unroll
             for (int px = 0; px < PX; px++) {
-                and_popc_acc(cp[px][o0 + g], a[px][j], wp);
-                and_popc_acc(cn[px][o0 + g], a[px][j], wn);
+                if (OR1) {
+                    cp[px][o0 + g] |= a[px][j] & wp;
+                    cn[px][o0 + g] |= a[px][j] & wn;
+                } else {
+                    and_popc_acc(cp[px][o0 + g], a[px][j], wp);
+                    and_popc_acc(cn[px][o0 + g], a[px][j], wn);
+                }
             }
         }
 }
@@ -104,12 +111,15 @@ constexpr int MAX_NS = 4; // waves per block (each takes a share of the stream s
 // s_waitcnt immediate: lgkmcnt(0), vmcnt and expcnt left at their maxima (not waited for)
 constexpr int WAIT_LGKM0 = 0xC07F;
 
-template <int KW, int ZC, int PX, int OT, bool WIDE>
+// MODE 0: 16-bit packed sums; 1 (WIDE): 32-bit sums for the linear op's large saturation values;
+// 2 (OR1): 16-bit packed sums with n_sat = 1, evaluated with and-or instead of and-popcount.
+template <int KW, int ZC, int PX, int OT, int MODE>
 __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t *__restrict__ A,
                                                         const uint32_t *__restrict__ Wst, ComputeParams p,
                                                         uint32_t *__restrict__ part, int16_t *__restrict__ out_pos,
                                                         int16_t *__restrict__ out_neg, int16_t *__restrict__ out_diff)
 {
+    constexpr bool WIDE = MODE == 1, OR1 = MODE == 2;
     constexpr int KWZ = KW * ZC;
     constexpr int BM = 64 * PX;            // pixels per block (every wave of the block covers all of them)
     __shared__ uint32_t s_red[MAX_NS][WIDE ? 2 : 1][PX * OT][64];
@@ -221,7 +231,7 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                 for (int e = 0; e < BW; e++) wb1[e] = src[e];
             }
             __builtin_amdgcn_sched_barrier(0); // keep the prefetch above the VALU work it overlaps with
-            compute_batch<PX, OT, KWZ, G>(a_cur, wb0, cp, cn, b * G);
+            compute_batch<PX, OT, KWZ, G, OR1>(a_cur, wb0, cp, cn, b * G);
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(WAIT_LGKM0);
             {
@@ -230,12 +240,18 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                 for (int e = 0; e < BW; e++) wb0[e] = src[e];
             }
             __builtin_amdgcn_sched_barrier(0);
-            compute_batch<PX, OT, KWZ, G>(a_cur, wb1, cp, cn, (b + 1) * G);
+            compute_batch<PX, OT, KWZ, G, OR1>(a_cur, wb1, cp, cn, (b + 1) * G);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (slot_done) {
             // per-slot saturation and accumulation
-            if (!WIDE) {
+            if (OR1) { // [any bit set], both for min(count, 1) and for count >= 1
+#pragma unroll
+                for (int px = 0; px < PX; px++)
+#pragma unroll
+                    for (int o = 0; o < OT; o++)
+                        acc[px][o] = pk_add_u16(acc[px][o], min(cp[px][o], 1u) | (min(cn[px][o], 1u) << 16));
+            } else if (!WIDE) {
                 if (p.mode == 0) {
 #pragma unroll
                     for (int px = 0; px < PX; px++)
@@ -457,7 +473,7 @@ __global__ __launch_bounds__(256) void sc_compute_generic_kernel(const uint32_t 
 }
 
 // ---- host side ---------------------------------------------------------------------------------
-template <int KW, int ZC, int PX, int OT, bool WIDE>
+template <int KW, int ZC, int PX, int OT, int MODE>
 static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams p, uint32_t *part, int16_t *out_pos,
                           int16_t *out_neg, int16_t *out_diff, hipStream_t stream)
 {
@@ -471,10 +487,10 @@ static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams 
     REXSC_CHECK_ARG(blocks < (1L << 30), "SC compute: grid too large (%ld blocks)", blocks);
     const int grid = (int)align_up((size_t)blocks, 8);
     static char name[64] = "";
-    if (!name[0]) snprintf(name, sizeof(name), "sc_compute<%d,%d,%d,%d,%d>", KW, ZC, PX, OT, (int)WIDE);
+    if (!name[0]) snprintf(name, sizeof(name), "sc_compute<%d,%d,%d,%d,%d>", KW, ZC, PX, OT, MODE);
     // algorithmic lane-ops: (and + popcount-accumulate) x 2 polarities per 32-channel word
     ProfScope prof(name, 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
-    hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, WIDE>), dim3(grid), dim3(64 * p.ns), 0, stream, A, Wst, p, part,
+    hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, MODE>), dim3(grid), dim3(64 * p.ns), 0, stream, A, Wst, p, part,
                        out_pos, out_neg, out_diff);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
@@ -494,15 +510,21 @@ int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, i
                uint32_t *part, int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, hipStream_t stream)
 {
     const int px = p.px;
+    // saturation at one: the and-or instances (not in WIDE mode, whose sums are not packed)
+    const bool or1 = !wide && (p.nn & 0xffffu) == 1u;
 #define REXSC_INST(KW_, ZC_)                                                                                      \
     if (KW == KW_ && ZC == ZC_) {                                                                                 \
-        if (px == 2) return launch_compute<KW_, ZC_, 2, 16, false>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
-        return launch_compute<KW_, ZC_, 1, 16, false>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);      \
+        if (or1) {                                                                                                \
+            if (px == 2) return launch_compute<KW_, ZC_, 2, 16, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
+            return launch_compute<KW_, ZC_, 1, 16, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);      \
+        }                                                                                                         \
+        if (px == 2) return launch_compute<KW_, ZC_, 2, 16, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
+        return launch_compute<KW_, ZC_, 1, 16, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);          \
     }
     if (wide) {
         REXSC_CHECK_ARG(KW == 1 && (ZC == 4 || ZC == 8), "wide accumulation is only built for 1x1 / linear shapes");
-        if (ZC == 4) return launch_compute<1, 4, 1, 16, true>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
-        return launch_compute<1, 8, 1, 16, true>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
+        if (ZC == 4) return launch_compute<1, 4, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
+        return launch_compute<1, 8, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
     }
     REXSC_INST(1, 1) REXSC_INST(1, 2) REXSC_INST(1, 4) REXSC_INST(1, 8)
     REXSC_INST(3, 1) REXSC_INST(3, 2) REXSC_INST(3, 4)
