@@ -8,6 +8,11 @@ with numpy arrays in place of tensors, so a parity test reads like a call of the
 
 compute_bias_std_coef restates utils_functional.py:900-949 in numpy (float64 statistics
 are NOT used: the reference works in float32 tensors, and so does this).
+
+Pinning: the conv / linear / fixed-conv functions against tests/golden/ref_cpu_ext.npz (written by
+the reference's compiled CPU extension), compute_bias_std_coef against tests/golden/ref_calib.npz
+(written by the reference's own Python function); the scalar float functions (OR-n, bias/noise,
+quantise) against closed forms in tests/test_oracle_invariants.py.
 """
 import ctypes
 import os

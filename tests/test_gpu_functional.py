@@ -169,3 +169,16 @@ def test_tinyconv_training_step(sync):
     if sync == 1:
         l2, _ = run()
         assert l1 == l2
+
+
+def test_calibration_fit_matches_reference_python_on_gpu():
+    """sc_functional.compute_bias_std_coef (statistics kernel + host fit) against the vectors written
+    by the reference's own function."""
+    import sc_functional as uf
+    from test_oracle_golden import check_calib_against_reference
+
+    def fit(or_n, bit, act, order):
+        b, s = uf.compute_bias_std_coef(or_n, torch.from_numpy(bit).cuda(), torch.from_numpy(act).cuda(), order)
+        return b.cpu().numpy(), s.cpu().numpy()
+
+    check_calib_against_reference(fit)

@@ -41,3 +41,37 @@ def test_fixed_golden(case):
     got = orc.conv2d_saturate(_data["fixed/%s/x" % n], _data["fixed/%s/w" % n], case["add_config"],
                               case["precision_in"], case["precision_out"], case["padding"], case["stride"])
     assert np.array_equal(got, _data["fixed/%s/y" % n])
+
+
+def _calib_cases():
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_calib.npz"))
+    return g, [c.split(",") for c in g["cases"]]
+
+
+def _poly_values(coef, xs):
+    return sum(float(coef[i]) * xs ** i for i in range(len(coef)))
+
+
+def check_calib_against_reference(fit):
+    """fit(or_n, a_bit, a_act, order) -> (bias_coef, std_coef) against the vectors written by the
+    reference's own compute_bias_std_coef (tests/golden/make_golden_calib.py).  The reference solves
+    its least-squares problems in float32, which leaves the coefficients of the ill-conditioned
+    power basis loose in the sixth digit; what is compared is the fitted polynomial over the
+    calibrated range, to 2e-5 of its magnitude."""
+    g, cases = _calib_cases()
+    for name, or_n, order in cases:
+        bit, act = g[name + "_bit"], g[name + "_act"]
+        b, s = fit(int(or_n), bit, act, int(order))
+        b, s = np.asarray(b, np.float64), np.asarray(s, np.float64)
+        assert b.shape == g[name + "_bias"].shape and s.shape == g[name + "_std"].shape
+        xs = np.linspace(0, float(bit.max()), 64)
+        for mine, ref in ((b, g[name + "_bias"]), (s, g[name + "_std"])):
+            want = _poly_values(ref, xs)
+            assert np.abs(_poly_values(mine, xs) - want).max() <= 2e-5 * np.abs(want).max() + 1e-7, name
+        # the suppression rule zeroes the bias fit exactly
+        if not g[name + "_bias"].any():
+            assert not b.any(), name
+
+
+def test_calibration_fit_matches_reference_python():
+    check_calib_against_reference(orc.compute_bias_std_coef)
