@@ -108,19 +108,33 @@ def config3_tinyconv_step(torch, dev):
 
 def config4_fixed_conv(torch, dev):
     import fixed_extension_cuda
-    out = {"workload": "saturating fixed-point conv forward (add_config 0, 5-bit operands, 24-bit accumulator), "
-                       "batch 64, conv3x3 s1 p1", "shapes": {}}
+    import sc_functional as uf
+    out = {"workload": "saturating fixed-point conv (add_config 0, 5-bit operands, 24-bit accumulator), batch 64, "
+                       "conv3x3 s1 p1: forward kernel alone, and forward + backward through the float conv", "shapes": {}}
     for C, H in ((64, 56), (128, 28), (256, 14), (512, 7)):
         g = torch.Generator().manual_seed(4)
         x = (torch.randint(0, 32, (64, C, H, H), generator=g).float() / 32).to(dev)
         w = (torch.randint(-31, 32, (C, C, 3, 3), generator=g).float() / 32).to(dev)
         fn = lambda: fixed_extension_cuda.conv2d_saturate_acc(x, w, 0, 5, 24, (1, 1), (1, 1))
         sec = _time(torch, fn, 10, 2)
+        # forward + backward as the training path runs it: fixed-point forward values over the float
+        # conv, whose backward supplies the gradients (generator 'fixed', forward 'full_bin')
+        xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        gout = torch.randn(64, C, H, H, generator=g).to(dev)
+
+        def fwd_bwd():
+            xg.grad = None
+            wg.grad = None
+            uf.conv2d_generic(xg, wg, (1, 1), (1, 1), bit_length=32, forward="full_bin", generator="fixed",
+                              sync=1).backward(gout)
+
+        sec_fb = _time(torch, fwd_bwd, 10, 3)
         nbytes = 4 * x.numel() + 4 * w.numel() + 4 * 64 * C * H * H
         mac = 64 * H * H * C * C * 9
         out["shapes"]["%dx%dx%d" % (C, H, H)] = {"ms": sec * 1e3, "GB_per_s": nbytes / sec / 1e9,
                                                "hbm_frac": nbytes / sec / HBM_PEAK, "mac_per_s": mac / sec,
-                                               "images_per_s": 64 / sec}
+                                               "images_per_s": 64 / sec, "forward_backward_ms": sec_fb * 1e3,
+                                               "images_per_s_fwd_bwd": 64 / sec_fb}
     return out
 
 
