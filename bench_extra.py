@@ -154,6 +154,33 @@ def config5_resnet18_step(torch, dev, batch=64):
     return res
 
 
+def resnet18_sc_conv_fwd_bwd(torch, dev, batch=64):
+    """The 19 SC conv layers of ResNet-18 through conv2d_generic (sync 1): integer SC forward over the
+    float OR-2 surrogate, backward through the surrogate (two float convs and the OR-n kernels)."""
+    import sc_functional as uf
+    from bench import RESNET18_SC_LAYERS, make_conv_operands
+    layers = []
+    for i, (C, H, O, K, s) in enumerate(RESNET18_SC_LAYERS):
+        x, w = make_conv_operands(torch, batch, C, H, O, K, 32, seed=900 + i)
+        x = x.to(dev).contiguous(memory_format=torch.channels_last).requires_grad_(True)
+        w = (w.to(dev) * 0.1).requires_grad_(True)
+        Ho = (H + 2 * (K // 2) - K) // s + 1
+        gout = torch.randn(batch, O, Ho, Ho, device=dev).contiguous(memory_format=torch.channels_last)
+        layers.append((x, w, K, s, gout))
+
+    def step():
+        for (x, w, K, s, gout) in layers:
+            x.grad = None
+            w.grad = None
+            uf.conv2d_generic(x, w, (K // 2, K // 2), (s, s), bit_length=32, forward="or_2", generator="lfsr",
+                              sync=1).backward(gout)
+
+    sec = _time(torch, step, 5, 2)
+    return {"workload": "19 ResNet-18 SC conv layers, batch %d, OR-2, 32-bit streams, channels_last: SC forward + "
+                        "backward through the float surrogate (conv2d_generic, sync 1)" % batch,
+            "ms_per_step": sec * 1e3, "images_per_s": batch / sec}
+
+
 def pointwise(torch, dev):
     import _ops
     n = 64 * 64 * 56 * 56  # one ResNet-18 layer1 activation tensor
@@ -176,7 +203,8 @@ def run(torch, dev):
     out = {}
     for name, fn in (("config1_sc_conv_or1", config1_sc_conv_or1), ("config2_sc_linear", config2_sc_linear),
                      ("config3_tinyconv_train", config3_tinyconv_step), ("config4_fixed_conv", config4_fixed_conv),
-                     ("config5_resnet18_train", config5_resnet18_step), ("pointwise", pointwise)):
+                     ("config5_resnet18_train", config5_resnet18_step),
+                     ("resnet18_sc_conv_fwd_bwd", resnet18_sc_conv_fwd_bwd), ("pointwise", pointwise)):
         try:
             out[name] = fn(torch, dev)
         except Exception as e:
