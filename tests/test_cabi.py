@@ -73,3 +73,26 @@ def test_ops_fail_loudly_without_the_library(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "missing.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.lib()
+
+
+def test_product_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing under the package, and none of the product's entry
+    modules, may import, load or run anything under oracle/ (bench.py may, for its CPU baseline only;
+    __graft_entry__ may, to build it and inside smoke())."""
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    pkg = os.path.join(root, "rex-sc_amd")
+    pat = re.compile(r"oracle|rexsc_oracle|_ref\b")
+    offenders = []
+    for dirpath, _, files in os.walk(pkg):
+        if os.path.basename(dirpath) in ("build", "__pycache__"):
+            continue
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f), encoding="utf-8", errors="replace").read()
+                for n, line in enumerate(text.splitlines(), 1):
+                    if pat.search(line) and "cpu_oracle" not in line:
+                        offenders.append("%s:%d: %s" % (os.path.relpath(os.path.join(dirpath, f), root), n, line.strip()))
+    assert not offenders, "\n".join(offenders)
+    extra = open(os.path.join(root, "bench_extra.py")).read()
+    assert "oracle" not in extra
