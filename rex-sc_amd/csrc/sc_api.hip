@@ -164,8 +164,8 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     // (256 CUs x 4 SIMDs x 3) so that its tail is short; what the tiles and NS do not supply comes
     // from splitting the slots over blocks as well (partials merged by the finalize kernel).
     const int o_tiles = O_pad / OT;
-    // REXSC_TUNE_PX_MIN_M (default 1024): fewest output pixels for which a lane takes two of them
-    cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 1024)) ? 2 : 1;
+    // REXSC_TUNE_PX_MIN_M (default 128): fewest output pixels for which a lane takes two of them
+    cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 128)) ? 2 : 1;
     cp.ns = n_slots >= 8 ? 4 : (n_slots >= 2 ? 2 : 1);
     const long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
     int splits = 1;
@@ -178,7 +178,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
         const double work1 = (double)ceil_div(n_slots, cp.ns) * KH * ZG * (4.0 * cp.px * OT * KW * ZC);
         const double overhead = tune_env("REXSC_TUNE_WAVE_OVERHEAD", 1500);
         double best = 0;
-        for (int s = 1; s <= max_splits && s <= 8; s *= 2) {
+        for (int s = 1; s <= max_splits && s <= 16; s *= 2) {
             const double rounds = (double)((waves * s + TARGET_WAVES - 1) / TARGET_WAVES);
             double cost = rounds * (work1 / s + overhead);
             if (s > 1) {
