@@ -12,6 +12,7 @@
 // (linear); quantisation sc_conv.cpp:316-320.
 #include <stdlib.h>
 #include <string.h>
+#include <type_traits>
 #include <utility>
 
 #include "sng.h"
@@ -584,7 +585,7 @@ static int sng_activations_sliced(const float *x, uint32_t *A, const uint32_t *T
 // Block: 256 threads, one (group of `wog` output channels, ky, zg); wog is 16, 8, 4 or 2, the largest
 // that still gives the launch several hundred blocks.
 constexpr int W_OG_MAX = 16;
-constexpr int W_SLOT_GROUP = 32; // upper bound; the launcher shrinks it to fit the LDS budget
+constexpr int W_SLOT_GROUP = 32; // upper bound (64 in the lane = slot variant); the launcher shrinks it to fit the LDS budget
 
 // s_waitcnt immediate: vmcnt(0), expcnt and lgkmcnt left at their maxima (not waited for)
 constexpr int WAIT_VM0 = 0x0F70;
@@ -598,7 +599,10 @@ constexpr int W_COMBO_CHUNK = 8; // (kx, 64-channel half) combinations whose sta
 //  * "value > state" for the 32 channels of a word is then 2 bitwise operations per plane, and
 //    the lane ends up with the finished stream word of (slot t, word w), which it puts into the
 //    staging row of slot t.
-template <int ZC, int LB, bool PROG>
+// S64: a group is 64 slots and lane = slot; the two words of a 64-channel half are finished one after
+// the other with the ballot halves as scalar operands (no per-lane select), and weights are loaded
+// and balloted once per 64 slots.  Otherwise a group is 32 slots and lane = (word, slot).
+template <int ZC, int LB, bool PROG, bool S64>
 __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict__ w, uint32_t *__restrict__ Wst,
                                                          const SeqTable *__restrict__ tables, WeightGeom geo, GenParams gp,
                                                          int slot_group, int wog, ActTableJob job)
@@ -609,8 +613,11 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
     uint8_t *s_seq = s_dyn;
     uint8_t *s_inv = s_dyn + SEQ_LEN;
     uint8_t *s_pos = s_dyn + SEQ_LEN + 256;                                 // [combo in chunk][channel of the half]
-    uint32_t *s_S = reinterpret_cast<uint32_t *>(s_pos + W_COMBO_CHUNK * 64); // [combo in chunk][plane 0..7][lane]
+    // [combo in chunk][word (S64 only)][plane 0..7][lane]: W_COMBO_CHUNK combinations, half as many for S64
+    uint32_t *s_S = reinterpret_cast<uint32_t *>(s_pos + W_COMBO_CHUNK * 64);
     uint32_t *s_stage = s_S + W_COMBO_CHUNK * 8 * 64;
+    constexpr int CCHUNK = S64 ? W_COMBO_CHUNK / 2 : W_COMBO_CHUNK;
+    constexpr int NW = S64 ? 2 : 1;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -623,7 +630,8 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
     const int row = wog * 2 * KW * ZC; // words per slot handled by this block
     const int pitch = row + 2;          // LDS row pitch (bank spreading for the per-slot writes)
     const float S = (float)gp.scale;
-    const int wsel = lane >> 5, t = lane & 31; // this lane's word of the 64-channel half, and slot of the group
+    // this lane's word of the 64-channel half (both words in turn for S64), and its slot of the group
+    const int wsel = S64 ? 0 : lane >> 5, t = S64 ? lane : lane & 31;
     const int ncombo = KW * HALVES;
     // weight element of (output channel o, channel c, ky, kx): o*o_stride + lane part + h*h_step + kx*kx_mul
     const long o_stride = (long)geo.C * geo.KH * KW;
@@ -639,11 +647,11 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
         const int ns = min(slot_group, gp.n_slots - s0);
         const int cyc = slot_cycle(gp, s0 + min(t, ns - 1));
         const int first_plane = PROG ? prog_shift(gp, cyc) : 0;
-        for (int combo0 = 0; combo0 < ncombo; combo0 += W_COMBO_CHUNK) {
-            const int ncc = min(W_COMBO_CHUNK, ncombo - combo0);
+        for (int combo0 = 0; combo0 < ncombo; combo0 += CCHUNK) {
+            const int ncc = min(CCHUNK, ncombo - combo0);
             // cycle position of every channel's seed, lane = channel of the 64-channel half:
             // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
-            if (s0 == 0 || ncombo > W_COMBO_CHUNK) {
+            if (s0 == 0 || ncombo > CCHUNK) {
                 for (int cl = wave; cl < ncc; cl += 4) {
                     const int combo = combo0 + cl;
                     const int h = combo % HALVES, kx = combo / HALVES;
@@ -655,17 +663,20 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
             }
             // state planes of this lane's (word, slot) for every combination of the chunk
             for (int cl = wave; cl < ncc; cl += 4) {
-                const uint8_t *pos = s_pos + cl * 64 + wsel * 32;
-                const uint8_t *seq = s_seq + 1 + cyc;
-                uint32_t R[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int cc = 0; cc < 32; cc++) {
-                    const uint32_t st = seq[pos[cc]];
-                    R[cc & 7] |= st << (8 * (cc >> 3));
+                for (int wq = 0; wq < NW; wq++) {
+                    const uint8_t *pos = s_pos + cl * 64 + (S64 ? wq : wsel) * 32;
+                    const uint8_t *seq = s_seq + 1 + cyc;
+                    uint32_t R[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                    for (int cc = 0; cc < 32; cc++) {
+                        const uint32_t st = seq[pos[cc]];
+                        R[cc & 7] |= st << (8 * (cc >> 3));
+                    }
+                    values_to_planes(R);
+#pragma unroll
+                    for (int k = 0; k < LB; k++) s_S[((cl * NW + wq) * 8 + k) * 64 + lane] = R[k];
                 }
-                values_to_planes(R);
-#pragma unroll
-                for (int k = 0; k < LB; k++) s_S[(cl * 8 + k) * 64 + lane] = R[k];
             }
             __syncthreads();
 
@@ -714,22 +725,32 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
                     // counts as negative, as it does in ceil(-clamp(f*S, 1-S, 0)).
                     const uint32_t mag = (uint32_t)(int)ceilf(fminf(fabsf(f * S), S - 1.f));
                     const unsigned long long neg = __ballot(!(f >= 0.f));
-                    uint32_t gt_p = 0, gt_n = 0;
+                    uint32_t gt_p[NW], gt_n[NW];
+#pragma unroll
+                    for (int wq = 0; wq < NW; wq++) { gt_p[wq] = 0; gt_n[wq] = 0; }
 #pragma unroll
                     for (int k = 0; k < LB; k++) {
                         const unsigned long long m = __ballot((mag >> k) & 1u);
                         const unsigned long long mp = m & ~neg, mn = m & neg;
-                        uint32_t vkp = wsel ? (uint32_t)(mp >> 32) : (uint32_t)mp;
-                        uint32_t vkn = wsel ? (uint32_t)(mn >> 32) : (uint32_t)mn;
-                        if (PROG && k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
-                        const uint32_t sk = s_S[(cl * 8 + k) * 64 + lane];
-                        const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
-                        gt_p = (dp & vkp) | (~dp & gt_p);
-                        gt_n = (dn & vkn) | (~dn & gt_n);
+#pragma unroll
+                        for (int wq = 0; wq < NW; wq++) {
+                            const bool hi = S64 ? wq == 1 : wsel != 0;
+                            uint32_t vkp = hi ? (uint32_t)(mp >> 32) : (uint32_t)mp;
+                            uint32_t vkn = hi ? (uint32_t)(mn >> 32) : (uint32_t)mn;
+                            if (PROG && k < first_plane) { vkp = 0; vkn = 0; } // progressive loading truncates low bits
+                            const uint32_t sk = s_S[((cl * NW + wq) * 8 + k) * 64 + lane];
+                            const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
+                            gt_p[wq] = (dp & vkp) | (~dp & gt_p[wq]);
+                            gt_n[wq] = (dn & vkn) | (~dn & gt_n[wq]);
+                        }
                     }
-                    if (t < ns && h * 2 + wsel < ZC) {
-                        s_stage[t * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2 + wsel] = gt_p;
-                        s_stage[t * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2 + wsel] = gt_n;
+#pragma unroll
+                    for (int wq = 0; wq < NW; wq++) {
+                        const int wd = S64 ? wq : wsel;
+                        if (t < ns && h * 2 + wd < ZC) {
+                            s_stage[t * pitch + ((ol * 2 + 0) * KW + kx) * ZC + h * 2 + wd] = gt_p[wq];
+                            s_stage[t * pitch + ((ol * 2 + 1) * KW + kx) * ZC + h * 2 + wd] = gt_n[wq];
+                        }
                     }
                 }
 #pragma unroll
@@ -795,25 +816,45 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
         REXSC_CHECK_ARG(entries < (1L << 31), "activation SNG: state table too large");
         REXSC_CHECK_ARG(job.gp.lb == gp.lb && job.gp.acc == gp.acc, "activation and weight generators use different LFSRs");
     }
-    const size_t row_bytes = sizeof(uint32_t) * (wog * 2 * geo.KW * ZC + 2);
     const size_t fixed = SEQ_LEN + 256 + W_COMBO_CHUNK * 64 + sizeof(uint32_t) * W_COMBO_CHUNK * 8 * 64;
+    auto row_bytes_of = [&](int g) { return sizeof(uint32_t) * (g * 2 * geo.KW * ZC + 2); };
+    // 64-slot groups (lane = slot) when the streams are long enough and 64 staging rows fit the LDS
+    // budget, if need be with fewer output channels per block
+    bool s64 = gp.n_slots >= 64;
+    if (s64) {
+        int g = wog;
+        while (g > 2 && fixed + row_bytes_of(g) * 64 > 60 * 1024) g /= 2;
+        if (fixed + row_bytes_of(g) * 64 <= 60 * 1024) wog = g; else s64 = false;
+    }
+    const long n_wblocks2 = (long)(geo.O_pad / wog) * geo.KH * geo.ZG; // wog may have shrunk
+    REXSC_CHECK_ARG(n_wblocks2 < (1L << 31), "weight SNG: grid too large");
+    const size_t row_bytes = row_bytes_of(wog);
     int slot_group = (int)((60 * 1024 - fixed) / row_bytes);
-    if (slot_group > W_SLOT_GROUP) slot_group = W_SLOT_GROUP;
+    const int group_cap = s64 ? 64 : W_SLOT_GROUP;
+    if (slot_group > group_cap) slot_group = group_cap;
     REXSC_CHECK_ARG(slot_group >= 1, "weight SNG: kernel width %d too large for LDS staging", geo.KW);
     const size_t lds = fixed + row_bytes * slot_group;
     ProfScope prof("sng_weight", 4.0 * geo.O * geo.C * geo.KH * geo.KW +
                                      4.0 * gp.n_slots * geo.KH * geo.ZG * geo.O_pad * 2 * geo.KW * ZC, stream);
     auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3((unsigned)n_wblocks), dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group, wog,
-                           job);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)n_wblocks2), dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group,
+                           wog, job);
+    };
+    auto launch_lb = [&](auto lb_tag) {
+        constexpr int LB = decltype(lb_tag)::value;
+        if (s64) {
+            if (gp.prog) launch(sng_weight_kernel<ZC, LB, true, true>); else launch(sng_weight_kernel<ZC, LB, false, true>);
+        } else {
+            if (gp.prog) launch(sng_weight_kernel<ZC, LB, true, false>); else launch(sng_weight_kernel<ZC, LB, false, false>);
+        }
     };
     switch (gp.lb) {
-    case 3: if (gp.prog) launch(sng_weight_kernel<ZC, 3, true>); else launch(sng_weight_kernel<ZC, 3, false>); break;
-    case 4: if (gp.prog) launch(sng_weight_kernel<ZC, 4, true>); else launch(sng_weight_kernel<ZC, 4, false>); break;
-    case 5: if (gp.prog) launch(sng_weight_kernel<ZC, 5, true>); else launch(sng_weight_kernel<ZC, 5, false>); break;
-    case 6: if (gp.prog) launch(sng_weight_kernel<ZC, 6, true>); else launch(sng_weight_kernel<ZC, 6, false>); break;
-    case 7: if (gp.prog) launch(sng_weight_kernel<ZC, 7, true>); else launch(sng_weight_kernel<ZC, 7, false>); break;
-    case 8: if (gp.prog) launch(sng_weight_kernel<ZC, 8, true>); else launch(sng_weight_kernel<ZC, 8, false>); break;
+    case 3: launch_lb(std::integral_constant<int, 3>{}); break;
+    case 4: launch_lb(std::integral_constant<int, 4>{}); break;
+    case 5: launch_lb(std::integral_constant<int, 5>{}); break;
+    case 6: launch_lb(std::integral_constant<int, 6>{}); break;
+    case 7: launch_lb(std::integral_constant<int, 7>{}); break;
+    case 8: launch_lb(std::integral_constant<int, 8>{}); break;
     default: set_error("weight SNG: unsupported LFSR width %d", gp.lb); return REXSC_ERR_INVALID;
     }
     REXSC_CHECK_HIP(hipGetLastError());
