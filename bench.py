@@ -76,6 +76,8 @@ def main():
     ap.add_argument("--cpu-sample-batch", type=int, default=64)
     ap.add_argument("--only-layer", default=None, metavar="C,H,O,K,S",
                     help="run a single SC conv layer shape instead of the 19 (for per-kernel counter runs)")
+    ap.add_argument("--only-extra", default=None, metavar="NAME",
+                    help="run one function of bench_extra.py (e.g. pointwise, config4_fixed_conv) and exit (for profiler runs)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run three 256 MiB device-to-device copies and exit (scales the rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -102,6 +104,14 @@ def main():
         torch.cuda.synchronize()
         return 0
     _lib.check(_lib.lib().rexsc_init(None), "rexsc_init")
+    if args.only_extra:
+        import bench_extra
+        fn = getattr(bench_extra, args.only_extra, None)  # a function of bench_extra.py, e.g. pointwise
+        if not callable(fn) or args.only_extra.startswith("_") or args.only_extra == "run":
+            print("bench.py: no configuration named %r in bench_extra.py" % args.only_extra, file=sys.stderr)
+            return 2
+        print(json.dumps({args.only_extra: fn(torch, dev)}))
+        return 0
 
     shapes = RESNET18_SC_LAYERS
     if args.only_layer:
