@@ -435,6 +435,47 @@ __global__ __launch_bounds__(256) void sc_finalize_kernel(const uint32_t *__rest
     }
 }
 
+// Finalize for channels-last int16 results with narrow (uint16) partials and O % 4 == 0: a thread sums
+// four adjacent output channels (one 8-byte load per split) and writes 8 bytes per tensor.
+__global__ __launch_bounds__(256) void sc_finalize_nhwc4_kernel(const uint32_t *__restrict__ part, ComputeParams p,
+                                                                int16_t *__restrict__ out_pos, int16_t *__restrict__ out_neg,
+                                                                int16_t *__restrict__ out_diff)
+{
+    const unsigned o4 = (unsigned)p.O / 4;
+    const unsigned total = (unsigned)p.M * o4;
+    const long split_stride = (long)p.O_pad * p.M; // in uint16 elements
+    const uint16_t *part16 = reinterpret_cast<const uint16_t *>(part);
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+        const unsigned m = i / o4, q = i - m * o4;
+        const long idx0 = (long)m * p.O_pad + q * 4;
+        uint32_t sp[4] = {0, 0, 0, 0}, sn[4] = {0, 0, 0, 0};
+        for (int s0 = 0; s0 < p.splits; s0 += 8) {
+            uint2 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                v[u] = make_uint2(0, 0);
+                if (s0 + u < p.splits) v[u] = *reinterpret_cast<const uint2 *>(part16 + idx0 + (long)(s0 + u) * split_stride);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                sp[0] += v[u].x & 0xffu; sn[0] += (v[u].x >> 8) & 0xffu;
+                sp[1] += (v[u].x >> 16) & 0xffu; sn[1] += v[u].x >> 24;
+                sp[2] += v[u].y & 0xffu; sn[2] += (v[u].y >> 8) & 0xffu;
+                sp[3] += (v[u].y >> 16) & 0xffu; sn[3] += v[u].y >> 24;
+            }
+        }
+        const long o_idx = (long)m * p.O + q * 4;
+        if (out_pos) *reinterpret_cast<uint2 *>(out_pos + o_idx) = make_uint2((sp[0] & 0xffffu) | (sp[1] << 16), (sp[2] & 0xffffu) | (sp[3] << 16));
+        if (out_neg) *reinterpret_cast<uint2 *>(out_neg + o_idx) = make_uint2((sn[0] & 0xffffu) | (sn[1] << 16), (sn[2] & 0xffffu) | (sn[3] << 16));
+        if (out_diff) {
+            uint32_t d[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) d[e] = (sp[e] - sn[e]) & 0xffffu;
+            *reinterpret_cast<uint2 *>(out_diff + o_idx) = make_uint2(d[0] | (d[1] << 16), d[2] | (d[3] << 16));
+        }
+    }
+}
+
 // Generic fallback for kernel widths without a tuned instance: one output per thread, runtime loops.
 __global__ __launch_bounds__(256) void sc_compute_generic_kernel(const uint32_t *__restrict__ A,
                                                                  const uint32_t *__restrict__ Wst, ComputeParams p,
@@ -553,7 +594,12 @@ int sc_finalize_i16(const uint32_t *part, const ComputeParams &p, int16_t *out_p
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
     ProfScope prof("sc_finalize_i16", (double)total * ((p.part_narrow ? 2.0 : 4.0) * p.splits + 4.0), stream);
-    if (total < (1L << 31))
+    const bool aligned8 = ((uintptr_t)out_pos % 8) == 0 && ((uintptr_t)out_neg % 8) == 0 && ((uintptr_t)out_diff % 8) == 0;
+    if (p.out_channels_last && p.part_narrow && p.O % 4 == 0 && aligned8 && total < (1L << 31)) {
+        const long t4 = total / 4;
+        const int grid4 = (int)((t4 + 255) / 256 < 16384 ? (t4 + 255) / 256 : 16384);
+        hipLaunchKernelGGL(sc_finalize_nhwc4_kernel, dim3(grid4), dim3(256), 0, stream, part, p, out_pos, out_neg, out_diff);
+    } else if (total < (1L << 31))
         hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
                            out_neg, out_diff);
     else
