@@ -125,6 +125,35 @@ int rexsc_orn_bias_std_forward_f16(const uint16_t *x_half, const float *bias_coe
 int rexsc_orn_bias_std_backward(const float *grad_out, const float *x, const float *bias_coef,
                                 float *grad_in, size_t n, int or_n, int half_input, rexsc_stream_t stream);
 
+/* ---- polarity-pair layout (merged surrogate convolution) ----------------------------------
+ * conv2d_generic evaluates its float surrogate as two convolutions, with clamp(w, 0, 100) and with
+ * -clamp(w, -100, 0) (utils_functional.py:1204-1211, 1249), and sends each sum through the OR-n
+ * kernels.  Convolving once with the 2*O filters [w_pos ; w_neg] yields the same sums as one tensor
+ * s2 laid out [outer][2][inner] float32 (channels-last: outer = N*Ho*Wo, inner = O; NCHW: outer = N,
+ * inner = O*Ho*Wo; linear: outer = B, inner = O); y and grad_out are [outer][inner].  inner % 4 == 0.
+ * rexsc_orn_pair_backward = two or_approx_n_backward_acc calls on (g, s_pos) and (-g, s_neg)
+ * (sc_cuda_pw.cu:767-832); the bias_std_pair calls = the *_both_acc calls above on this layout, with
+ * the same noise stream per element of y.  g2 has s2's layout (gradient of the merged convolution). */
+int rexsc_orn_pair_backward(const float *grad_out, const float *s2, float *g2, size_t outer, size_t inner,
+                            int or_n, int half_input, rexsc_stream_t stream);
+int rexsc_orn_bias_std_pair_forward(const float *s2, const float *bias_coef, const float *std_coef, float *y,
+                                    size_t outer, size_t inner, int or_n, uint64_t seed, uint64_t offset,
+                                    rexsc_stream_t stream);
+int rexsc_orn_bias_std_pair_backward(const float *grad_out, const float *s2, const float *bias_coef, float *g2,
+                                     size_t outer, size_t inner, int or_n, int half_input,
+                                     rexsc_stream_t stream);
+
+/* y = float(pos) / bit_length - float(neg) / bit_length over n elements of any dense layout: the
+ * int16 -> float, "/ bit_length" and "pos - neg" passes of utils_functional.py:1181-1182, 1273-1274
+ * and 1317 in one. */
+int rexsc_sc_counts_to_float(const int16_t *pos, const int16_t *neg, float *y, size_t n, int bit_length,
+                             rexsc_stream_t stream);
+
+/* w2[0..n) = clamp(w, 0, 100), w2[n..2n) = -clamp(w, -100, 0) (utils_functional.py:1204-1205), and the
+ * gradient of that split: dw = dw2[0..n) * [0 <= w <= 100] - dw2[n..2n) * [-100 <= w <= 0]. */
+int rexsc_split_weight(const float *w, float *w2, size_t n, rexsc_stream_t stream);
+int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t n, rexsc_stream_t stream);
+
 /* Philox4x32-10 block function on the host (for known-answer tests of the generator). */
 void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
 

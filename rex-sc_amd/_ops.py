@@ -198,14 +198,22 @@ def orn_backward(grad_output, x, or_n, half_input=True):
 _philox = {"seed": None, "offset": 0}
 
 
-def _next_philox(n_elems):
-    """(seed, offset) for the next noise draw: the seed follows torch.manual_seed, the offset
-    advances by the number of 4-element vectors consumed."""
+def _next_philox(n_elems, device):
+    """(seed, offset) for the next noise draw, taken from the device's torch generator and advanced
+    past the 4-element vectors this call consumes -- the way the reference's kernels consume the
+    generator's Philox state (sc_cuda_pw.cu:870-877): torch.manual_seed restarts the stream.  While a
+    stream is being captured the generator may not be touched; a counter of this module stands in."""
+    used = (n_elems + 3) // 4
+    if not torch.cuda.is_current_stream_capturing():
+        gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+        seed, off = gen.initial_seed() & 0xFFFFFFFFFFFFFFFF, gen.get_offset()
+        gen.set_offset(off + (used + 3) // 4 * 4)  # the generator keeps offsets in multiples of 4
+        return seed, off
     seed = torch.initial_seed() & 0xFFFFFFFFFFFFFFFF
     if _philox["seed"] != seed:
         _philox["seed"], _philox["offset"] = seed, 0
     off = _philox["offset"]
-    _philox["offset"] = off + (n_elems + 3) // 4
+    _philox["offset"] = off + used
     return seed, off
 
 
@@ -217,7 +225,7 @@ def orn_bias_std_both_forward(x_pos, x_neg, bias_coef, std_coef, or_n, seed=None
     y = torch.empty_like(xp)
     n = xp.numel()
     if seed is None:
-        seed, offset = _next_philox(n)
+        seed, offset = _next_philox(n, xp.device)
     np_ = torch.empty_like(xp) if return_noise else None
     nn_ = torch.empty_like(xp) if return_noise else None
     with torch.cuda.device(xp.device):
@@ -246,7 +254,7 @@ def orn_bias_std_forward_f16(x, bias_coef, std_coef, or_n, seed=None, offset=Non
     b, s = _coef(bias_coef, xh.device), _coef(std_coef, xh.device)
     y = torch.empty_like(xh)
     if seed is None:
-        seed, offset = _next_philox(xh.numel())
+        seed, offset = _next_philox(xh.numel(), xh.device)
     with torch.cuda.device(xh.device):
         rc = _lib.lib().rexsc_orn_bias_std_forward_f16(_ptr(xh), _ptr(b), _ptr(s), _ptr(y), xh.numel(), int(or_n),
                                                        int(seed), int(offset), _stream())
@@ -265,6 +273,113 @@ def orn_bias_std_backward(grad_output, x, bias_coef, or_n, half_input=True):
                                                     int(half_input), _stream())
         _lib.check(rc, "rexsc_orn_bias_std_backward")
     return gx
+
+
+# ---- merged surrogate (polarity-pair layout) ---------------------------------------------------
+
+def pair_layout(s2):
+    """s2 = conv / linear output with 2*O channels (O positive, then O negative).  Returns
+    (s2 dense, outer, inner, channels_last) for the [outer][2][inner] view of its storage, re-laying
+    the tensor out if its own layout has no inner % 4 == 0 view; None if neither layout has one."""
+    s2 = s2.detach()
+    O = s2.size(1) // 2
+    if s2.dim() == 2:
+        return (s2.contiguous(), s2.size(0), O, False) if O % 4 == 0 else None
+    N, _, H, W = s2.shape
+    ok_cl, ok_nchw = O % 4 == 0, (O * H * W) % 4 == 0
+    is_cl = s2.is_contiguous(memory_format=torch.channels_last) and not s2.is_contiguous()
+    if (is_cl and ok_cl) or (not ok_nchw and ok_cl):
+        return _as_layout(s2, True), N * H * W, O, True
+    if ok_nchw:
+        return _as_layout(s2, False), N, O * H * W, False
+    return None
+
+
+def _pair_result_like(s2, channels_last):
+    if s2.dim() == 2:
+        return torch.empty((s2.size(0), s2.size(1) // 2), dtype=torch.float32, device=s2.device)
+    N, O2, H, W = s2.shape
+    return _empty_out((N, O2 // 2, H, W), torch.float32, s2.device, channels_last)
+
+
+def orn_pair_backward(grad_output, s2, outer, inner, channels_last, or_n, half_input=True):
+    y_like = _pair_result_like(s2, channels_last)
+    g = _like_layout(grad_output, y_like)
+    g2 = torch.empty_like(s2)
+    with torch.cuda.device(s2.device):
+        rc = _lib.lib().rexsc_orn_pair_backward(_ptr(g), _ptr(s2), _ptr(g2), outer, inner, int(or_n), int(half_input),
+                                                _stream())
+        _lib.check(rc, "rexsc_orn_pair_backward")
+    return g2
+
+
+def orn_bias_std_pair_forward(s2, outer, inner, channels_last, bias_coef, std_coef, or_n, seed=None, offset=None):
+    b, s = _coef(bias_coef, s2.device), _coef(std_coef, s2.device)
+    y = _pair_result_like(s2, channels_last)
+    if seed is None:
+        seed, offset = _next_philox(y.numel(), y.device)
+    with torch.cuda.device(s2.device):
+        rc = _lib.lib().rexsc_orn_bias_std_pair_forward(_ptr(s2), _ptr(b), _ptr(s), _ptr(y), outer, inner, int(or_n),
+                                                        int(seed), int(offset), _stream())
+        _lib.check(rc, "rexsc_orn_bias_std_pair_forward")
+    return y
+
+
+def orn_bias_std_pair_backward(grad_output, s2, outer, inner, channels_last, bias_coef, or_n, half_input=True):
+    y_like = _pair_result_like(s2, channels_last)
+    g = _like_layout(grad_output, y_like)
+    b = _coef(bias_coef, s2.device)
+    g2 = torch.empty_like(s2)
+    with torch.cuda.device(s2.device):
+        rc = _lib.lib().rexsc_orn_bias_std_pair_backward(_ptr(g), _ptr(s2), _ptr(b), _ptr(g2), outer, inner, int(or_n),
+                                                         int(half_input), _stream())
+        _lib.check(rc, "rexsc_orn_bias_std_pair_backward")
+    return g2
+
+
+def sc_counts_to_float(pos, neg, bit_length):
+    """float(pos) / L - float(neg) / L in pos's layout (pos, neg: the int16 results of one SC conv call)."""
+    _require_cuda(pos, neg)
+    if pos.dtype != torch.int16 or neg.dtype != torch.int16 or pos.stride() != neg.stride():
+        raise RuntimeError("sc_counts_to_float: expected two int16 tensors of one layout")
+    y = torch.empty_like(pos, dtype=torch.float32)
+    if y.stride() != pos.stride():
+        raise RuntimeError("sc_counts_to_float: the SC result is not dense")
+    with torch.cuda.device(pos.device):
+        rc = _lib.lib().rexsc_sc_counts_to_float(_ptr(pos), _ptr(neg), _ptr(y), pos.numel(), int(bit_length),
+                                                 _stream())
+        _lib.check(rc, "rexsc_sc_counts_to_float")
+    return y
+
+
+def split_weight(w):
+    """[clamp(w, 0, 100) ; -clamp(w, -100, 0)] along dim 0, in w's (dense) memory order."""
+    _require_cuda(w)
+    wd = _dense_f32(w)
+    shape = (2 * wd.size(0),) + tuple(wd.shape[1:])
+    w2 = torch.empty_strided(shape, wd.stride(), dtype=torch.float32, device=wd.device)
+    with torch.cuda.device(wd.device):
+        rc = _lib.lib().rexsc_split_weight(_ptr(wd), _ptr(w2), wd.numel(), _stream())
+        _lib.check(rc, "rexsc_split_weight")
+    return w2
+
+
+def merge_weight_grad(dw2, w):
+    """Gradient with respect to w of split_weight, given the gradient of its result."""
+    wd = _dense_f32(w)
+    d2 = dw2.detach()
+    shape = (2 * wd.size(0),) + tuple(wd.shape[1:])
+    if tuple(d2.shape) != shape:
+        raise RuntimeError("merge_weight_grad: gradient shape %s does not match %s" % (tuple(d2.shape), shape))
+    if d2.dtype != torch.float32 or d2.stride() != wd.stride() or d2.data_ptr() % 16:
+        t = torch.empty_strided(shape, wd.stride(), dtype=torch.float32, device=wd.device)
+        t.copy_(d2)
+        d2 = t
+    dw = torch.empty_like(wd)
+    with torch.cuda.device(wd.device):
+        rc = _lib.lib().rexsc_merge_weight_grad(_ptr(d2), _ptr(wd), _ptr(dw), wd.numel(), _stream())
+        _lib.check(rc, "rexsc_merge_weight_grad")
+    return dw
 
 
 def calib_stats(a_bit, a_act, win_lo, win_hi):

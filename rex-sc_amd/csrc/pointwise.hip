@@ -278,6 +278,141 @@ __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_backward_kernel(const
         gx[i] = orn_bias_bwd<N>(g[i], half_input ? round_half(x[i]) : x[i], b);
 }
 
+// ---- polarity-pair layout ------------------------------------------------------------------------
+// The float surrogate of an SC layer can convolve with the positive and the negative weight parts in
+// one call (2*O output channels: the O positive ones, then the O negative ones).  Its sums then lie
+// in memory as [outer][2][inner] float32 -- channels-last conv output: outer = N*Ho*Wo, inner = O;
+// NCHW: outer = N, inner = O*Ho*Wo; linear: outer = B, inner = O -- while the layer's result and its
+// incoming gradient are [outer][inner].  These kernels read and write the pair layout in place of
+// two separate tensors; inner is a multiple of 4 (whole float4 vectors), q counts float4 vectors of
+// the [outer][inner] tensor and the noise stream is indexed by q exactly as in the two-tensor kernels.
+__device__ __forceinline__ size_t pair_vec_offset(size_t q, unsigned inner4)
+{
+    const unsigned o = (unsigned)q / inner4; // the host checks that q fits 32 bits
+    return (size_t)q + (size_t)o * inner4;   // = o * 2 * inner4 + (q - o * inner4)
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_pair_backward_kernel(const float *__restrict__ g,
+                                                                       const float *__restrict__ s2,
+                                                                       float *__restrict__ g2, size_t nvec,
+                                                                       unsigned inner4, int half_input)
+{
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        const size_t off = pair_vec_offset(q, inner4);
+        float4 a = reinterpret_cast<const float4 *>(s2)[off];
+        float4 c = reinterpret_cast<const float4 *>(s2)[off + inner4];
+        const float4 gg = reinterpret_cast<const float4 *>(g)[q];
+        if (half_input) {
+            a.x = round_half(a.x); a.y = round_half(a.y); a.z = round_half(a.z); a.w = round_half(a.w);
+            c.x = round_half(c.x); c.y = round_half(c.y); c.z = round_half(c.z); c.w = round_half(c.w);
+        }
+        float4 rp, rn;
+        rp.x = orn_bwd<N>(gg.x, a.x); rn.x = orn_bwd<N>(-gg.x, c.x);
+        rp.y = orn_bwd<N>(gg.y, a.y); rn.y = orn_bwd<N>(-gg.y, c.y);
+        rp.z = orn_bwd<N>(gg.z, a.z); rn.z = orn_bwd<N>(-gg.z, c.z);
+        rp.w = orn_bwd<N>(gg.w, a.w); rn.w = orn_bwd<N>(-gg.w, c.w);
+        reinterpret_cast<float4 *>(g2)[off] = rp;
+        reinterpret_cast<float4 *>(g2)[off + inner4] = rn;
+    }
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_bias_std_pair_forward_kernel(
+    const float *__restrict__ s2, const float *__restrict__ bc, const float *__restrict__ sc, float *__restrict__ y,
+    size_t nvec, unsigned inner4, uint64_t seed, uint64_t offset)
+{
+    const Coef6 b = load_coef(bc), s = load_coef(sc);
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        float zp[4], zn[4];
+        normal4(seed, offset + q, 0u, zp);
+        normal4(seed, offset + q, 1u, zn);
+        const size_t off = pair_vec_offset(q, inner4);
+        const float4 a = reinterpret_cast<const float4 *>(s2)[off];
+        const float4 c = reinterpret_cast<const float4 *>(s2)[off + inner4];
+        float4 r;
+        r.x = bias_noise_fwd(orn_fwd<N>(a.x), zp[0], b, s) - bias_noise_fwd(orn_fwd<N>(c.x), zn[0], b, s);
+        r.y = bias_noise_fwd(orn_fwd<N>(a.y), zp[1], b, s) - bias_noise_fwd(orn_fwd<N>(c.y), zn[1], b, s);
+        r.z = bias_noise_fwd(orn_fwd<N>(a.z), zp[2], b, s) - bias_noise_fwd(orn_fwd<N>(c.z), zn[2], b, s);
+        r.w = bias_noise_fwd(orn_fwd<N>(a.w), zp[3], b, s) - bias_noise_fwd(orn_fwd<N>(c.w), zn[3], b, s);
+        reinterpret_cast<float4 *>(y)[q] = r;
+    }
+}
+
+template <int N>
+__global__ __launch_bounds__(PW_THREADS) void orn_bias_std_pair_backward_kernel(
+    const float *__restrict__ g, const float *__restrict__ s2, const float *__restrict__ bc, float *__restrict__ g2,
+    size_t nvec, unsigned inner4, int half_input)
+{
+    const Coef6 b = load_coef(bc);
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        const size_t off = pair_vec_offset(q, inner4);
+        float4 a = reinterpret_cast<const float4 *>(s2)[off];
+        float4 c = reinterpret_cast<const float4 *>(s2)[off + inner4];
+        const float4 gg = reinterpret_cast<const float4 *>(g)[q];
+        if (half_input) {
+            a.x = round_half(a.x); a.y = round_half(a.y); a.z = round_half(a.z); a.w = round_half(a.w);
+            c.x = round_half(c.x); c.y = round_half(c.y); c.z = round_half(c.z); c.w = round_half(c.w);
+        }
+        float4 rp, rn;
+        rp.x = orn_bias_bwd<N>(gg.x, a.x, b); rn.x = orn_bias_bwd<N>(-gg.x, c.x, b);
+        rp.y = orn_bias_bwd<N>(gg.y, a.y, b); rn.y = orn_bias_bwd<N>(-gg.y, c.y, b);
+        rp.z = orn_bias_bwd<N>(gg.z, a.z, b); rn.z = orn_bias_bwd<N>(-gg.z, c.z, b);
+        rp.w = orn_bias_bwd<N>(gg.w, a.w, b); rn.w = orn_bias_bwd<N>(-gg.w, c.w, b);
+        reinterpret_cast<float4 *>(g2)[off] = rp;
+        reinterpret_cast<float4 *>(g2)[off + inner4] = rn;
+    }
+}
+
+// SC result as the layer's float output: y = pos / L - neg / L (utils_functional.py:1181-1182, 1273-1274, 1317).
+// torch divides a tensor by a Python scalar as a multiplication by the scalar's float reciprocal; so does this.
+__global__ __launch_bounds__(PW_THREADS) void sc_counts_to_float_kernel(const int16_t *__restrict__ pos,
+                                                                        const int16_t *__restrict__ neg,
+                                                                        float *__restrict__ y, size_t n, float inv_L)
+{
+    const size_t nvec = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        const uint2 p = reinterpret_cast<const uint2 *>(pos)[q];
+        const uint2 m = reinterpret_cast<const uint2 *>(neg)[q];
+        float4 r;
+        r.x = (float)(int16_t)(p.x & 0xffffu) * inv_L - (float)(int16_t)(m.x & 0xffffu) * inv_L;
+        r.y = (float)(int16_t)(p.x >> 16) * inv_L - (float)(int16_t)(m.x >> 16) * inv_L;
+        r.z = (float)(int16_t)(p.y & 0xffffu) * inv_L - (float)(int16_t)(m.y & 0xffffu) * inv_L;
+        r.w = (float)(int16_t)(p.y >> 16) * inv_L - (float)(int16_t)(m.y >> 16) * inv_L;
+        reinterpret_cast<float4 *>(y)[q] = r;
+    }
+    const size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = (float)pos[i] * inv_L - (float)neg[i] * inv_L;
+}
+
+// w2 = [clamp(w, 0, 100) ; -clamp(w, -100, 0)]  (utils_functional.py:1204-1205)
+__global__ __launch_bounds__(PW_THREADS) void split_weight_kernel(const float *__restrict__ w, float *__restrict__ w2,
+                                                                  size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = w[i];
+    w2[i] = v != v ? v : fminf(fmaxf(v, 0.f), 100.f); // clamp keeps NaN, as torch's does
+    w2[n + i] = v != v ? v : -fminf(fmaxf(v, -100.f), 0.f);
+}
+
+// Gradient of the two clamps: each passes its incoming gradient where w lies inside its closed range.
+__global__ __launch_bounds__(PW_THREADS) void merge_weight_grad_kernel(const float *__restrict__ dw2,
+                                                                       const float *__restrict__ w,
+                                                                       float *__restrict__ dw, size_t n)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float v = w[i];
+    const float gp = (v >= 0.f && v <= 100.f) ? dw2[i] : 0.f;
+    const float gn = (v >= -100.f && v <= 0.f) ? dw2[n + i] : 0.f;
+    dw[i] = gp - gn;
+}
+
 // Calibration statistics: per window k, count / sum / sum of squares of (a_bit - a_act) over
 // the elements with lo[k] <= a_act < hi[k].  Windows may overlap.
 constexpr int CAL_MAX_WIN = 64;
@@ -477,6 +612,107 @@ extern "C" int rexsc_calib_stats(const float *a_bit, const float *a_act, size_t 
     const int grid = (int)(tiles < 4096 ? tiles : 4096);
     ProfScope prof("calib_stats", 8.0 * n, stream);
     hipLaunchKernelGGL(calib_stats_kernel, dim3(grid), dim3(256), 0, stream, a_bit, a_act, n, w, n_win, stats);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+// ---- polarity-pair entry points ----------------------------------------------------------------------
+static int check_pair(size_t outer, size_t inner)
+{
+    REXSC_CHECK_ARG(inner % 4 == 0, "pair layout needs inner %% 4 == 0 (got %zu)", inner);
+    REXSC_CHECK_ARG(outer * inner / 4 < (1ull << 32), "pair layout: tensor too large (%zu x %zu)", outer, inner);
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_pair_backward(const float *g, const float *s2, float *g2, size_t outer, size_t inner, int or_n,
+                                       int half_input, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    if (int rc = check_pair(outer, inner)) return rc;
+    const size_t nvec = outer * inner / 4;
+    if (nvec == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(g && s2 && g2, "null pointer");
+    const int grid = pw_grid(nvec);
+    ProfScope prof("orn_pair_backward", 20.0 * outer * inner, stream);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_pair_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0, stream, g,
+                                               s2, g2, nvec, (unsigned)(inner / 4), half_input));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_bias_std_pair_forward(const float *s2, const float *bias_coef, const float *std_coef, float *y,
+                                               size_t outer, size_t inner, int or_n, uint64_t seed, uint64_t offset,
+                                               rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    if (int rc = check_pair(outer, inner)) return rc;
+    const size_t nvec = outer * inner / 4;
+    if (nvec == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(s2 && y && bias_coef && std_coef, "null pointer");
+    const int grid = pw_grid(nvec);
+    ProfScope prof("orn_bias_std_pair_forward", 12.0 * outer * inner, stream);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_pair_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
+                                               stream, s2, bias_coef, std_coef, y, nvec, (unsigned)(inner / 4), seed,
+                                               offset));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_orn_bias_std_pair_backward(const float *g, const float *s2, const float *bias_coef, float *g2,
+                                                size_t outer, size_t inner, int or_n, int half_input,
+                                                rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    if (int rc = check_pair(outer, inner)) return rc;
+    const size_t nvec = outer * inner / 4;
+    if (nvec == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(g && s2 && g2 && bias_coef, "null pointer");
+    const int grid = pw_grid(nvec);
+    ProfScope prof("orn_bias_std_pair_backward", 20.0 * outer * inner, stream);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_pair_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
+                                               stream, g, s2, bias_coef, g2, nvec, (unsigned)(inner / 4), half_input));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_sc_counts_to_float(const int16_t *pos, const int16_t *neg, float *y, size_t n, int bit_length,
+                                        rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(bit_length >= 1, "bit_length must be positive (got %d)", bit_length);
+    if (n == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(pos && neg && y, "null pointer");
+    const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("sc_counts_to_float", 8.0 * n, stream);
+    hipLaunchKernelGGL(sc_counts_to_float_kernel, dim3(grid), dim3(PW_THREADS), 0, stream, pos, neg, y, n,
+                       1.0f / (float)bit_length);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_split_weight(const float *w, float *w2, size_t n, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(w && w2, "null pointer");
+    REXSC_CHECK_ARG(n < (1ull << 31) * PW_THREADS, "tensor too large");
+    hipLaunchKernelGGL(split_weight_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS), 0,
+                       stream, w, w2, n);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t n, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    if (n == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(dw2 && w && dw, "null pointer");
+    REXSC_CHECK_ARG(n < (1ull << 31) * PW_THREADS, "tensor too large");
+    hipLaunchKernelGGL(merge_weight_grad_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS),
+                       0, stream, dw2, w, dw, n);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

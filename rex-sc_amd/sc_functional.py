@@ -208,6 +208,76 @@ def compute_bias_std_coef(or_n, a_bit, a_act, order):
     return torch.from_numpy(bias_coef).to(dev), torch.from_numpy(std_coef).to(dev)
 
 
+# ---- merged surrogate ---------------------------------------------------------------------------
+class Merged_Surrogate_Conv(torch.autograd.Function):
+    """The float surrogate of conv2d_generic for forward = 'or_n' (n <= 4) / 'full_or' with its two
+    convolutions merged: one conv with the 2*O filters [clamp(w, 0, 100) ; -clamp(w, -100, 0)]
+    (utils_functional.py:1204-1211), the OR-n / error-injection kernels reading both halves of its
+    output in place, one backward conv pair for both polarities.
+
+    sync = 1: the forward value is the SC result `sc_value` (= pos / L - neg / L, the tensor the
+    reference writes into `.data`, :1273-1274) and the OR-n forward is never evaluated;
+    sync = 3: the forward value is the fused OR-n + bias/noise kernel's (:1253-1254).
+    Gradients are those of OR_n(conv(x, w_pos)) - OR_n(conv(x, w_neg)) (sync 3: with the bias
+    polynomial's derivative), evaluated on the saved sums rounded to binary16 as the reference's
+    backward wrappers do."""
+
+    @staticmethod
+    def forward(ctx, activation, weight, sc_value, bias_coef, std_coef, or_n, pad_hw, stride, sync):
+        w2 = _ops.split_weight(weight)
+        s2, outer, inner, cl = _ops.pair_layout(F.conv2d(activation, w2, padding=pad_hw, stride=stride))
+        ctx.geom = (outer, inner, cl, or_n, tuple(pad_hw), tuple(stride), sync)
+        if sync == 3:
+            ctx.save_for_backward(activation, weight, s2, bias_coef)
+            return _ops.orn_bias_std_pair_forward(s2, outer, inner, cl, bias_coef, std_coef, or_n)
+        ctx.save_for_backward(activation, weight, s2)
+        return sc_value
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        outer, inner, cl, or_n, pad_hw, stride, sync = ctx.geom
+        if sync == 3:
+            activation, weight, s2, bias_coef = ctx.saved_tensors
+            g2 = _ops.orn_bias_std_pair_backward(grad_output, s2, outer, inner, cl, bias_coef, or_n)
+        else:
+            activation, weight, s2 = ctx.saved_tensors
+            g2 = _ops.orn_pair_backward(grad_output, s2, outer, inner, cl, or_n)
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        dx = dw = None
+        if need_x or need_w:
+            w2 = _ops.split_weight(weight)
+            dx, dw2, _ = torch.ops.aten.convolution_backward(g2, activation, w2, None, stride, pad_hw, (1, 1), False,
+                                                             (0, 0), 1, (need_x, need_w, False))
+            if need_w:
+                dw = _ops.merge_weight_grad(dw2, weight).to(weight.dtype)
+        return dx, dw, None, None, None, None, None, None, None
+
+
+def _merged_surrogate_ok(activation, weight, forward, or_n, sync, sc_on, split_output, stride, pad_hw):
+    """Whether conv2d_generic may take the merged path: float32 operands on the GPU, OR-n with a
+    fused kernel, a plain forward value (no split output), and an output shape with a whole number
+    of float4 vectors per polarity block.  REXSC_MERGED_SURROGATE=0 switches it off."""
+    if os.environ.get("REXSC_MERGED_SURROGATE", "1") == "0" or split_output or torch.is_autocast_enabled():
+        return False
+    if not (activation.is_cuda and weight.is_cuda) or activation.dtype != torch.float32 or weight.dtype != torch.float32:
+        return False
+    if sync == 1:
+        if not sc_on or not (forward in ("full_or", "and_2") or (forward[:3] == "or_" and len(forward) == 4)):
+            return False
+    elif sync == 3:
+        if not (forward[:3] == "or_" and len(forward) == 4):
+            return False
+    else:
+        return False
+    n = 1 if forward in ("full_or", "and_2") else or_n
+    if not 1 <= n <= 4:
+        return False
+    O, _, KH, KW = weight.shape
+    Ho = (activation.size(2) + 2 * pad_hw[0] - KH) // stride[0] + 1
+    Wo = (activation.size(3) + 2 * pad_hw[1] - KW) // stride[1] + 1
+    return O % 4 == 0 or (O * Ho * Wo) % 4 == 0
+
+
 # ---- generic SC layers ------------------------------------------------------------------------
 def _parse_forward(forward, generator):
     """forward / generator strings -> (or_n, bin_config, gen_config) (utils_functional.py:1160-1178)."""
@@ -263,6 +333,21 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     or_n, bin_config, gen_config = _parse_forward(forward, generator)
     global_sync = os.environ.get("Global_Sync", "1") == "1"
     sc_on = global_sync and (not Use_Approx) and 0 < sync_override < 3
+
+    stride = (int(stride[0]), int(stride[1]))
+    has_sc_kernel = bin_config is not None and gen_config is not None
+    if (sync_override == 3 or has_sc_kernel) and _merged_surrogate_ok(
+            activation, weight, forward, or_n, sync_override, sc_on, split_output, stride, pad_hw):
+        n = 1 if forward in ("full_or", "and_2") else or_n
+        sc_value = None
+        if sync_override == 1:
+            with torch.no_grad():
+                pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(
+                    activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
+                    (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
+                sc_value = _ops.sc_counts_to_float(pos, neg, bit_length)
+        return Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride,
+                                           sync_override)
 
     result_pos = result_neg = None
     if sc_on:

@@ -1,0 +1,121 @@
+"""conv2d_generic with the two surrogate convolutions merged (polarity-pair layout) against the
+two-convolution path it replaces: forward values, gradients, noise stream, layouts, fallbacks."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _operands(seed, N, C, H, W, O, K, L=32, dens=0.4):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randint(0, L, (N, C, H, W), generator=g).float() / L) * (torch.rand(N, C, H, W, generator=g) < dens)
+    w = (torch.randint(-L + 1, L, (O, C, K, K), generator=g).float() / L) * (torch.rand(O, C, K, K, generator=g) < dens)
+    return x, w
+
+
+def _run(monkeypatch, merged, x, w, pad, stride, forward, sync, channels_last, need_x=True, seed=11, bias=None,
+         std=None):
+    import sc_functional as uf
+    monkeypatch.setenv("REXSC_MERGED_SURROGATE", "1" if merged else "0")
+    xt = x.cuda()
+    if channels_last:
+        xt = xt.contiguous(memory_format=torch.channels_last)
+    xt.requires_grad_(need_x)
+    wt = w.cuda().requires_grad_(True)
+    torch.manual_seed(seed)
+    kw = dict(bit_length=32, generator="lfsr", forward=forward, sync=sync, order=5)
+    if bias is not None:
+        kw.update(bias_coef=bias.cuda(), std_coef=std.cuda())
+    out = uf.conv2d_generic(xt, wt, pad, stride, **kw)
+    g = torch.randn(out.shape, generator=torch.Generator().manual_seed(5)).cuda()
+    out.backward(g)
+    return out.detach().cpu(), (xt.grad.cpu() if need_x else None), wt.grad.cpu()
+
+
+def _close(a, b, what):
+    scale = float(b.abs().max()) + 1e-30
+    err = float((a - b).abs().max())
+    assert err <= 1e-5 * scale, "%s: max error %g against scale %g" % (what, err, scale)
+
+
+CASES = [
+    # N, C, H, W, O, K, pad, stride, channels_last
+    (2, 16, 10, 10, 12, 3, (1, 1), (1, 1), False),
+    (2, 16, 10, 10, 12, 3, (1, 1), (1, 1), True),
+    (3, 24, 9, 7, 8, 3, (1, 1), (2, 2), True),
+    (2, 8, 8, 8, 6, 1, (0, 0), (1, 1), False),     # O % 4 != 0, O*Ho*Wo % 4 == 0: NCHW pair layout
+    (2, 8, 8, 8, 6, 1, (0, 0), (1, 1), True),      # channels-last sums re-laid out as NCHW
+    (1, 40, 12, 12, 20, 5, (2, 2), (1, 1), True),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("forward", ["or_2", "or_3", "full_or"])
+def test_sync1_merged_equals_two_convolutions(case, forward, monkeypatch):
+    N, C, H, W, O, K, pad, stride, cl = case
+    print("merged sync1", case, forward, flush=True)
+    x, w = _operands(21, N, C, H, W, O, K)
+    ya, gxa, gwa = _run(monkeypatch, True, x, w, pad, stride, forward, 1, cl)
+    yb, gxb, gwb = _run(monkeypatch, False, x, w, pad, stride, forward, 1, cl)
+    assert torch.equal(ya, yb)   # the SC result, exactly
+    _close(gxa, gxb, "grad x")
+    _close(gwa, gwb, "grad w")
+
+
+@pytest.mark.parametrize("case", CASES[:4])
+def test_sync3_merged_equals_two_convolutions(case, monkeypatch):
+    N, C, H, W, O, K, pad, stride, cl = case
+    print("merged sync3", case, flush=True)
+    x, w = _operands(22, N, C, H, W, O, K)
+    bias = torch.tensor([0.01, -0.02, 0.005, 0.001, 0, 0])
+    std = torch.tensor([0.02, 0.01, 0, 0, 0, 0])
+    ya, gxa, gwa = _run(monkeypatch, True, x, w, pad, stride, "or_2", 3, cl, bias=bias, std=std)
+    yb, gxb, gwb = _run(monkeypatch, False, x, w, pad, stride, "or_2", 3, cl, bias=bias, std=std)
+    # same seed, same element order: the same noise draws, so the values agree to float rounding
+    _close(ya, yb, "forward")
+    _close(gxa, gxb, "grad x")
+    _close(gwa, gwb, "grad w")
+
+
+def test_first_layer_needs_no_activation_gradient(monkeypatch):
+    x, w = _operands(23, 2, 16, 8, 8, 8, 3)
+    ya, gxa, gwa = _run(monkeypatch, True, x, w, (1, 1), (1, 1), "or_2", 1, True, need_x=False)
+    yb, gxb, gwb = _run(monkeypatch, False, x, w, (1, 1), (1, 1), "or_2", 1, True, need_x=False)
+    assert gxa is None and torch.equal(ya, yb)
+    _close(gwa, gwb, "grad w")
+
+
+def test_shapes_without_a_vector_view_fall_back(monkeypatch):
+    # O = 5 and 5*3*3 = 45 outputs per image: no inner % 4 == 0 view in either layout
+    import sc_functional as uf
+    x, w = _operands(24, 2, 8, 3, 3, 5, 1)
+    calls = []
+    orig = uf.Merged_Surrogate_Conv.apply
+    monkeypatch.setattr(uf.Merged_Surrogate_Conv, "apply", lambda *a: calls.append(1) or orig(*a))
+    ya, gxa, gwa = _run(monkeypatch, True, x, w, (0, 0), (1, 1), "or_2", 1, False)
+    assert not calls
+    x2, w2 = _operands(24, 2, 8, 3, 3, 8, 1)
+    _run(monkeypatch, True, x2, w2, (0, 0), (1, 1), "or_2", 1, False)
+    assert calls
+
+
+def test_weight_split_and_merge_follow_clamp(monkeypatch):
+    import _ops
+    w = torch.tensor([-200.0, -100.0, -0.5, 0.0, 0.25, 100.0, 150.0, float("nan")]).reshape(8, 1, 1, 1).cuda()
+    w2 = _ops.split_weight(w)
+    want = torch.cat([w.clamp(0, 100), -(w.clamp(-100, 0))])
+    assert torch.equal(torch.nan_to_num(w2, nan=7.0), torch.nan_to_num(want, nan=7.0))
+    wr = w.clone().requires_grad_(True)
+    d2 = torch.arange(1.0, 17.0).reshape(16, 1, 1, 1).cuda()
+    torch.cat([wr.clamp(0, 100), -(wr.clamp(-100, 0))]).backward(d2)
+    assert torch.equal(_ops.merge_weight_grad(d2, w), wr.grad)
+
+
+def test_counts_to_float_odd_length():
+    import _ops
+    g = torch.Generator().manual_seed(3)
+    pos = torch.randint(-32768, 32767, (3, 5, 7, 3), generator=g, dtype=torch.int16).cuda()
+    neg = torch.randint(-32768, 32767, (3, 5, 7, 3), generator=g, dtype=torch.int16).cuda()
+    for L in (32, 48):
+        assert torch.equal(_ops.sc_counts_to_float(pos, neg, L), pos.float() / L - neg.float() / L)

@@ -152,3 +152,20 @@ def test_calib_stats_kernel():
         # float32 throughout): 1e-6 of the sum of magnitudes
         assert abs(st[k, 1] - err.sum()) <= 1e-6 * np.abs(err).sum() + 1e-9
         assert np.isclose(st[k, 2], (err * err).sum(), rtol=1e-6, atol=1e-9)
+
+
+def test_noise_stream_follows_the_torch_generator():
+    """Seed and offset come from the device's torch generator: re-seeding restarts the noise,
+    consecutive calls draw from disjoint parts of the stream."""
+    import sc_extension_cuda
+    x = torch.rand(5000, device="cuda")
+    coef0 = torch.zeros(6, device="cuda")
+    std = torch.tensor([0.5, 0, 0, 0, 0, 0], device="cuda")
+    torch.manual_seed(7)
+    a = sc_extension_cuda.or_approx_n_forward_bias_std_both_acc(x, x, coef0, std, 2)
+    b = sc_extension_cuda.or_approx_n_forward_bias_std_both_acc(x, x, coef0, std, 2)
+    torch.manual_seed(7)
+    c = sc_extension_cuda.or_approx_n_forward_bias_std_both_acc(x, x, coef0, std, 2)
+    assert torch.equal(a, c)
+    assert not torch.equal(a, b)
+    assert abs(float(((a - b) / 0.5).var()) - 4.0) < 0.4   # four independent N(0,1) draws per element
