@@ -346,6 +346,8 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
                     activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
                     (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
                 sc_value = _ops.sc_counts_to_float(pos, neg, bit_length)
+            if not (torch.is_grad_enabled() and (activation.requires_grad or weight.requires_grad)):
+                return sc_value  # inference: the surrogate only ever supplies gradients
         return Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride,
                                            sync_override)
 

@@ -119,3 +119,18 @@ def test_counts_to_float_odd_length():
     neg = torch.randint(-32768, 32767, (3, 5, 7, 3), generator=g, dtype=torch.int16).cuda()
     for L in (32, 48):
         assert torch.equal(_ops.sc_counts_to_float(pos, neg, L), pos.float() / L - neg.float() / L)
+
+
+def test_inference_skips_the_surrogate(monkeypatch):
+    """Without gradients sync 1 returns the SC result and never runs the float convolution."""
+    import sc_functional as uf
+    import torch.nn.functional as F
+    x, w = _operands(25, 2, 16, 8, 8, 8, 3)
+    xt, wt = x.cuda(), w.cuda().requires_grad_(True)
+    want = uf.conv2d_generic(xt, wt, (1, 1), (1, 1), bit_length=32, generator="lfsr", forward="or_2", sync=1).detach()
+    calls = []
+    orig = F.conv2d
+    monkeypatch.setattr(uf.F, "conv2d", lambda *a, **k: calls.append(1) or orig(*a, **k))
+    with torch.no_grad():
+        got = uf.conv2d_generic(xt, wt, (1, 1), (1, 1), bit_length=32, generator="lfsr", forward="or_2", sync=1)
+    assert torch.equal(got, want) and not calls and not got.requires_grad
