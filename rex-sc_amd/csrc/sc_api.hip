@@ -167,6 +167,10 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     // REXSC_TUNE_PX_MIN_M (default 128): fewest output pixels for which a lane takes two of them
     cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 128)) ? 2 : 1;
     cp.ns = n_slots >= 8 ? 4 : (n_slots >= 2 ? 2 : 1);
+    {
+        const int forced_ns = tune_env("REXSC_TUNE_NS", 0); // 1, 2 or 4 waves per block (tuning only)
+        if ((forced_ns == 1 || forced_ns == 2 || forced_ns == 4) && forced_ns <= n_slots) cp.ns = forced_ns;
+    }
     const long waves = (long)ceil_div(cp.M, 64 * cp.px) * cp.ns * o_tiles;
     int splits = 1;
     if (pl.tuned) {
@@ -175,7 +179,9 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
         // a fixed cost per wave (prologue, LDS reduction, stores).  Powers of two keep the shares even.
         // REXSC_TUNE_WAVE_OVERHEAD: that fixed cost in VALU instructions; REXSC_TUNE_SPLITS forces s.
         const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
-        const double work1 = (double)ceil_div(n_slots, cp.ns) * KH * ZG * (4.0 * cp.px * OT * KW * ZC);
+        // saturation at one needs one and-or per word and polarity instead of and + popcount
+        const double ops_per_word = (n_sat == 1 && !pl.wide) ? 2.0 : 4.0;
+        const double work1 = (double)ceil_div(n_slots, cp.ns) * KH * ZG * (ops_per_word * cp.px * OT * KW * ZC);
         const double overhead = tune_env("REXSC_TUNE_WAVE_OVERHEAD", 1500);
         double best = 0;
         for (int s = 1; s <= max_splits && s <= 16; s *= 2) {
