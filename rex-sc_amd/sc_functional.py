@@ -253,6 +253,20 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
         return dx, dw, None, None, None, None, None, None, None
 
 
+_side_streams = {}
+
+
+def _side_stream(device):
+    """Second stream (default priority) of a device for the SC forward, or None when overlap is
+    switched off (REXSC_OVERLAP_SURROGATE=0) or the caller's stream is being captured."""
+    if os.environ.get("REXSC_OVERLAP_SURROGATE", "1") == "0" or torch.cuda.is_current_stream_capturing():
+        return None
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _side_streams:
+        _side_streams[idx] = torch.cuda.Stream(device=idx)
+    return _side_streams[idx]
+
+
 def _merged_surrogate_ok(activation, weight, forward, or_n, sync, sc_on, split_output, stride, pad_hw):
     """Whether conv2d_generic may take the merged path: float32 operands on the GPU, OR-n with a
     fused kernel, a plain forward value (no split output), and an output shape with a whole number
@@ -339,17 +353,33 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     if (sync_override == 3 or has_sc_kernel) and _merged_surrogate_ok(
             activation, weight, forward, or_n, sync_override, sc_on, split_output, stride, pad_hw):
         n = 1 if forward in ("full_or", "and_2") else or_n
-        sc_value = None
-        if sync_override == 1:
+        if sync_override != 1:
+            return Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride,
+                                               sync_override)
+
+        def sc_forward():
             with torch.no_grad():
                 pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(
                     activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
                     (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
-                sc_value = _ops.sc_counts_to_float(pos, neg, bit_length)
-            if not (torch.is_grad_enabled() and (activation.requires_grad or weight.requires_grad)):
-                return sc_value  # inference: the surrogate only ever supplies gradients
-        return Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride,
-                                           sync_override)
+                return _ops.sc_counts_to_float(pos, neg, bit_length)
+
+        if not (torch.is_grad_enabled() and (activation.requires_grad or weight.requires_grad)):
+            return sc_forward()  # inference: the surrogate only ever supplies gradients
+        # The integer kernels (VALU-bound) and the surrogate's float convolution (matrix cores) are
+        # independent: the SC forward runs on a second stream of default priority and the two overlap.
+        side = _side_stream(activation.device)
+        if side is None:
+            return Merged_Surrogate_Conv.apply(activation, weight, sc_forward(), bias_coef, std_coef, n, pad_hw,
+                                               stride, 1)
+        cur = torch.cuda.current_stream(activation.device)
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            sc_value = sc_forward()
+        out = Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride, 1)
+        cur.wait_stream(side)
+        sc_value.record_stream(cur)  # allocated on the side stream, consumed on the caller's
+        return out
 
     result_pos = result_neg = None
     if sc_on:

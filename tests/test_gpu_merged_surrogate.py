@@ -134,3 +134,13 @@ def test_inference_skips_the_surrogate(monkeypatch):
     with torch.no_grad():
         got = uf.conv2d_generic(xt, wt, (1, 1), (1, 1), bit_length=32, generator="lfsr", forward="or_2", sync=1)
     assert torch.equal(got, want) and not calls and not got.requires_grad
+
+
+def test_side_stream_overlap_changes_nothing(monkeypatch):
+    """The SC forward on a second stream (default) and on the caller's stream give the same step."""
+    x, w = _operands(26, 4, 32, 14, 14, 32, 3)
+    monkeypatch.setenv("REXSC_OVERLAP_SURROGATE", "1")
+    ya, gxa, gwa = _run(monkeypatch, True, x, w, (1, 1), (1, 1), "or_2", 1, True)
+    monkeypatch.setenv("REXSC_OVERLAP_SURROGATE", "0")
+    yb, gxb, gwb = _run(monkeypatch, True, x, w, (1, 1), (1, 1), "or_2", 1, True)
+    assert torch.equal(ya, yb) and torch.equal(gxa, gxb) and torch.equal(gwa, gwb)
