@@ -149,10 +149,15 @@ int rexsc_orn_bias_std_pair_backward(const float *grad_out, const float *s2, con
 int rexsc_sc_counts_to_float(const int16_t *pos, const int16_t *neg, float *y, size_t n, int bit_length,
                              rexsc_stream_t stream);
 
-/* w2[0..n) = clamp(w, 0, 100), w2[n..2n) = -clamp(w, -100, 0) (utils_functional.py:1204-1205), and the
- * gradient of that split: dw = dw2[0..n) * [0 <= w <= 100] - dw2[n..2n) * [-100 <= w <= 0]. */
-int rexsc_split_weight(const float *w, float *w2, size_t n, rexsc_stream_t stream);
-int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t n, rexsc_stream_t stream);
+/* w2 = [clamp(w, 0, 100) ; -clamp(w, -100, 0)] along the output-channel axis (utils_functional.py:1204-1205)
+ * for w = [out_channels][in_channels][taps] (taps = KH*KW; 1 for a linear layer), and the gradient of that
+ * split: dw = dw2[first half] * [0 <= w <= 100] - dw2[second half] * [-100 <= w <= 0].  Each tensor is
+ * dense in one of two memory orders, named by its *_channels_last flag: [O][C][taps] (0) or [O][taps][C] (1);
+ * w2 can so be produced directly in the order a channels-last convolution wants.  dw has w's order. */
+int rexsc_split_weight(const float *w, float *w2, size_t out_channels, size_t in_channels, size_t taps,
+                       int w_channels_last, int w2_channels_last, rexsc_stream_t stream);
+int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t out_channels, size_t in_channels,
+                            size_t taps, int dw2_channels_last, int w_channels_last, rexsc_stream_t stream);
 
 /* Philox4x32-10 block function on the host (for known-answer tests of the generator). */
 void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);

@@ -352,32 +352,50 @@ def sc_counts_to_float(pos, neg, bit_length):
     return y
 
 
-def split_weight(w):
-    """[clamp(w, 0, 100) ; -clamp(w, -100, 0)] along dim 0, in w's (dense) memory order."""
-    _require_cuda(w)
+def _weight_geometry(w):
+    """(dense float32 w, O, C, taps, channels_last) of a conv [O,C,KH,KW] or linear [O,C] weight."""
     wd = _dense_f32(w)
-    shape = (2 * wd.size(0),) + tuple(wd.shape[1:])
-    w2 = torch.empty_strided(shape, wd.stride(), dtype=torch.float32, device=wd.device)
+    if wd.dim() == 2:
+        return wd, wd.size(0), wd.size(1), 1, False
+    O, C, KH, KW = wd.shape
+    cl = not wd.is_contiguous()  # _dense_f32 leaves only the two dense orders
+    return wd, O, C, KH * KW, cl
+
+
+def _empty_weight(O, C, KH, KW, channels_last, device):
+    if channels_last:
+        return torch.empty((O, KH, KW, C), dtype=torch.float32, device=device).permute(0, 3, 1, 2)
+    return torch.empty((O, C, KH, KW), dtype=torch.float32, device=device)
+
+
+def split_weight(w, channels_last=None):
+    """[clamp(w, 0, 100) ; -clamp(w, -100, 0)] along dim 0.  channels_last: memory order of the result
+    (None: w's own), so that a channels-last convolution needs no filter conversion."""
+    _require_cuda(w)
+    wd, O, C, taps, w_cl = _weight_geometry(w)
+    out_cl = w_cl if channels_last is None or wd.dim() == 2 else bool(channels_last)
+    if wd.dim() == 2:
+        w2 = torch.empty((2 * O, C), dtype=torch.float32, device=wd.device)
+    else:
+        w2 = _empty_weight(2 * O, C, wd.size(2), wd.size(3), out_cl, wd.device)
     with torch.cuda.device(wd.device):
-        rc = _lib.lib().rexsc_split_weight(_ptr(wd), _ptr(w2), wd.numel(), _stream())
+        rc = _lib.lib().rexsc_split_weight(_ptr(wd), _ptr(w2), O, C, taps, int(w_cl), int(out_cl), _stream())
         _lib.check(rc, "rexsc_split_weight")
     return w2
 
 
 def merge_weight_grad(dw2, w):
-    """Gradient with respect to w of split_weight, given the gradient of its result."""
-    wd = _dense_f32(w)
-    d2 = dw2.detach()
-    shape = (2 * wd.size(0),) + tuple(wd.shape[1:])
-    if tuple(d2.shape) != shape:
-        raise RuntimeError("merge_weight_grad: gradient shape %s does not match %s" % (tuple(d2.shape), shape))
-    if d2.dtype != torch.float32 or d2.stride() != wd.stride() or d2.data_ptr() % 16:
-        t = torch.empty_strided(shape, wd.stride(), dtype=torch.float32, device=wd.device)
-        t.copy_(d2)
-        d2 = t
+    """Gradient with respect to w of split_weight, given the gradient of its result (any dense order)."""
+    wd, O, C, taps, w_cl = _weight_geometry(w)
+    shape = (2 * O,) + tuple(wd.shape[1:])
+    if tuple(dw2.shape) != shape:
+        raise RuntimeError("merge_weight_grad: gradient shape %s does not match %s" % (tuple(dw2.shape), shape))
+    d2 = _dense_f32(dw2)
+    d2_cl = d2.dim() == 4 and not d2.is_contiguous()
     dw = torch.empty_like(wd)
     with torch.cuda.device(wd.device):
-        rc = _lib.lib().rexsc_merge_weight_grad(_ptr(d2), _ptr(wd), _ptr(dw), wd.numel(), _stream())
+        rc = _lib.lib().rexsc_merge_weight_grad(_ptr(d2), _ptr(wd), _ptr(dw), O, C, taps, int(d2_cl), int(w_cl),
+                                                _stream())
         _lib.check(rc, "rexsc_merge_weight_grad")
     return dw
 

@@ -389,27 +389,44 @@ __global__ __launch_bounds__(PW_THREADS) void sc_counts_to_float_kernel(const in
     if (i < n) y[i] = (float)pos[i] * inv_L - (float)neg[i] * inv_L;
 }
 
-// w2 = [clamp(w, 0, 100) ; -clamp(w, -100, 0)]  (utils_functional.py:1204-1205)
-__global__ __launch_bounds__(PW_THREADS) void split_weight_kernel(const float *__restrict__ w, float *__restrict__ w2,
-                                                                  size_t n)
+// w2 = [clamp(w, 0, 100) ; -clamp(w, -100, 0)]  (utils_functional.py:1204-1205).  w is [O][inner] with
+// inner = C*KH*KW in either memory order (src_cl: [KH*KW][C], else [C][KH*KW]); w2 is written in the
+// order dst_cl names, so that a channels-last convolution gets its filters without a conversion pass.
+__device__ __forceinline__ size_t weight_index(size_t i, unsigned inner, unsigned C, unsigned taps, bool from_cl, bool to_cl)
 {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    // index of element i (counted in `from` order) in `to` order
+    if (from_cl == to_cl) return i;
+    const size_t o = i / inner;
+    const unsigned r = (unsigned)(i - o * inner);
+    unsigned c, t;
+    if (from_cl) { t = r / C; c = r - t * C; } else { c = r / taps; t = r - c * taps; }
+    return o * inner + (to_cl ? t * C + c : c * taps + t);
+}
+
+__global__ __launch_bounds__(PW_THREADS) void split_weight_kernel(const float *__restrict__ w, float *__restrict__ w2,
+                                                                  size_t n, unsigned C, unsigned taps, int src_cl,
+                                                                  int dst_cl)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; // in w2's order
     if (i >= n) return;
-    const float v = w[i];
+    const float v = w[weight_index(i, C * taps, C, taps, dst_cl != 0, src_cl != 0)];
     w2[i] = v != v ? v : fminf(fmaxf(v, 0.f), 100.f); // clamp keeps NaN, as torch's does
     w2[n + i] = v != v ? v : -fminf(fmaxf(v, -100.f), 0.f);
 }
 
 // Gradient of the two clamps: each passes its incoming gradient where w lies inside its closed range.
+// dw is written in w's order (w_cl), dw2 is read in its own (dw2_cl).
 __global__ __launch_bounds__(PW_THREADS) void merge_weight_grad_kernel(const float *__restrict__ dw2,
                                                                        const float *__restrict__ w,
-                                                                       float *__restrict__ dw, size_t n)
+                                                                       float *__restrict__ dw, size_t n, unsigned C,
+                                                                       unsigned taps, int dw2_cl, int w_cl)
 {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; // in w's order
     if (i >= n) return;
+    const size_t j = weight_index(i, C * taps, C, taps, w_cl != 0, dw2_cl != 0);
     const float v = w[i];
-    const float gp = (v >= 0.f && v <= 100.f) ? dw2[i] : 0.f;
-    const float gn = (v >= -100.f && v <= 0.f) ? dw2[n + i] : 0.f;
+    const float gp = (v >= 0.f && v <= 100.f) ? dw2[j] : 0.f;
+    const float gn = (v >= -100.f && v <= 0.f) ? dw2[n + j] : 0.f;
     dw[i] = gp - gn;
 }
 
@@ -693,26 +710,32 @@ extern "C" int rexsc_sc_counts_to_float(const int16_t *pos, const int16_t *neg, 
     return REXSC_OK;
 }
 
-extern "C" int rexsc_split_weight(const float *w, float *w2, size_t n, rexsc_stream_t stream_)
+extern "C" int rexsc_split_weight(const float *w, float *w2, size_t out_channels, size_t in_channels, size_t taps,
+                                  int w_channels_last, int w2_channels_last, rexsc_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
+    const size_t n = out_channels * in_channels * taps;
     if (n == 0) return REXSC_OK;
     REXSC_CHECK_ARG(w && w2, "null pointer");
-    REXSC_CHECK_ARG(n < (1ull << 31) * PW_THREADS, "tensor too large");
+    REXSC_CHECK_ARG(in_channels * taps < (1ull << 32) && n < (1ull << 31) * PW_THREADS, "tensor too large");
     hipLaunchKernelGGL(split_weight_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS), 0,
-                       stream, w, w2, n);
+                       stream, w, w2, n, (unsigned)in_channels, (unsigned)taps, w_channels_last, w2_channels_last);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
 
-extern "C" int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t n, rexsc_stream_t stream_)
+extern "C" int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t out_channels,
+                                       size_t in_channels, size_t taps, int dw2_channels_last, int w_channels_last,
+                                       rexsc_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
+    const size_t n = out_channels * in_channels * taps;
     if (n == 0) return REXSC_OK;
     REXSC_CHECK_ARG(dw2 && w && dw, "null pointer");
-    REXSC_CHECK_ARG(n < (1ull << 31) * PW_THREADS, "tensor too large");
+    REXSC_CHECK_ARG(in_channels * taps < (1ull << 32) && n < (1ull << 31) * PW_THREADS, "tensor too large");
     hipLaunchKernelGGL(merge_weight_grad_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS),
-                       0, stream, dw2, w, dw, n);
+                       0, stream, dw2, w, dw, n, (unsigned)in_channels, (unsigned)taps, dw2_channels_last,
+                       w_channels_last);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

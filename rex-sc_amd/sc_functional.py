@@ -224,28 +224,28 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, activation, weight, sc_value, bias_coef, std_coef, or_n, pad_hw, stride, sync):
-        w2 = _ops.split_weight(weight)
+        # the filters are written in the activation's memory order: no conversion pass inside the convolutions
+        w2 = _ops.split_weight(weight, channels_last=_ops.is_channels_last(activation))
         s2, outer, inner, cl = _ops.pair_layout(F.conv2d(activation, w2, padding=pad_hw, stride=stride))
         ctx.geom = (outer, inner, cl, or_n, tuple(pad_hw), tuple(stride), sync)
         if sync == 3:
-            ctx.save_for_backward(activation, weight, s2, bias_coef)
+            ctx.save_for_backward(activation, weight, w2, s2, bias_coef)
             return _ops.orn_bias_std_pair_forward(s2, outer, inner, cl, bias_coef, std_coef, or_n)
-        ctx.save_for_backward(activation, weight, s2)
+        ctx.save_for_backward(activation, weight, w2, s2)
         return sc_value
 
     @staticmethod
     def backward(ctx, grad_output):
         outer, inner, cl, or_n, pad_hw, stride, sync = ctx.geom
         if sync == 3:
-            activation, weight, s2, bias_coef = ctx.saved_tensors
+            activation, weight, w2, s2, bias_coef = ctx.saved_tensors
             g2 = _ops.orn_bias_std_pair_backward(grad_output, s2, outer, inner, cl, bias_coef, or_n)
         else:
-            activation, weight, s2 = ctx.saved_tensors
+            activation, weight, w2, s2 = ctx.saved_tensors
             g2 = _ops.orn_pair_backward(grad_output, s2, outer, inner, cl, or_n)
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         dx = dw = None
         if need_x or need_w:
-            w2 = _ops.split_weight(weight)
             dx, dw2, _ = torch.ops.aten.convolution_backward(g2, activation, w2, None, stride, pad_hw, (1, 1), False,
                                                              (0, 0), 1, (need_x, need_w, False))
             if need_w:

@@ -112,6 +112,26 @@ def test_weight_split_and_merge_follow_clamp(monkeypatch):
     assert torch.equal(_ops.merge_weight_grad(d2, w), wr.grad)
 
 
+@pytest.mark.parametrize("w_cl", [False, True])
+@pytest.mark.parametrize("out_cl", [False, True])
+def test_weight_split_and_merge_in_both_memory_orders(w_cl, out_cl):
+    import _ops
+    g = torch.Generator().manual_seed(9)
+    w = (torch.rand(6, 5, 3, 2, generator=g) * 2 - 1).cuda()
+    if w_cl:
+        w = w.contiguous(memory_format=torch.channels_last)
+    w2 = _ops.split_weight(w, channels_last=out_cl)
+    assert w2.is_contiguous(memory_format=torch.channels_last if out_cl else torch.contiguous_format)
+    assert torch.equal(w2, torch.cat([w.clamp(0, 100), -(w.clamp(-100, 0))]))
+    d2 = torch.randn(12, 5, 3, 2, generator=g).cuda()
+    if out_cl:
+        d2 = d2.contiguous(memory_format=torch.channels_last)
+    wr = w.clone().requires_grad_(True)
+    torch.cat([wr.clamp(0, 100), -(wr.clamp(-100, 0))]).backward(d2)
+    got = _ops.merge_weight_grad(d2, w)
+    assert got.stride() == w.stride() and torch.equal(got, wr.grad)
+
+
 def test_counts_to_float_odd_length():
     import _ops
     g = torch.Generator().manual_seed(3)
@@ -143,4 +163,6 @@ def test_side_stream_overlap_changes_nothing(monkeypatch):
     ya, gxa, gwa = _run(monkeypatch, True, x, w, (1, 1), (1, 1), "or_2", 1, True)
     monkeypatch.setenv("REXSC_OVERLAP_SURROGATE", "0")
     yb, gxb, gwb = _run(monkeypatch, True, x, w, (1, 1), (1, 1), "or_2", 1, True)
-    assert torch.equal(ya, yb) and torch.equal(gxa, gxb) and torch.equal(gwa, gwb)
+    assert torch.equal(ya, yb)
+    _close(gxa, gxb, "grad x")   # MIOpen's gradient kernels accumulate with atomics: not bit-reproducible
+    _close(gwa, gwb, "grad w")
