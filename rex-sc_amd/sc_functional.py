@@ -253,6 +253,28 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
         return dx, dw, None, None, None, None, None, None, None
 
 
+class Merged_Surrogate_Linear(torch.autograd.Function):
+    """The same for the linear op: one GEMM with the 2*O rows [w_pos ; w_neg]; the forward value is the
+    SC result, the gradient that of OR_n(x w_pos^T) - OR_n(x w_neg^T) on the binary16-rounded sums."""
+
+    @staticmethod
+    def forward(ctx, activation, weight, sc_value, or_n):
+        w2 = _ops.split_weight(weight)
+        s2, outer, inner, _ = _ops.pair_layout(F.linear(activation, w2))
+        ctx.geom = (outer, inner, or_n)
+        ctx.save_for_backward(activation, w2, weight, s2)
+        return sc_value
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        outer, inner, or_n = ctx.geom
+        activation, w2, weight, s2 = ctx.saved_tensors
+        g2 = _ops.orn_pair_backward(grad_output, s2, outer, inner, False, or_n)
+        dx = g2 @ w2 if ctx.needs_input_grad[0] else None
+        dw = _ops.merge_weight_grad(g2.t() @ activation, weight).to(weight.dtype) if ctx.needs_input_grad[1] else None
+        return dx, dw, None, None
+
+
 _side_streams = {}
 
 
@@ -468,6 +490,19 @@ def linear_generic_sc(activation, weight, **kwargs):
     or_n, bin_config, gen_config = _parse_forward(forward, generator)
     if bin_config is None or gen_config is None:
         raise ValueError("linear_generic_sc: unsupported forward=%r / generator=%r" % (forward, generator))
+    merged = (os.environ.get("REXSC_MERGED_SURROGATE", "1") != "0" and sync_override == 1 and forward != "full_bin"
+              and 1 <= (or_n if or_n > 0 else 1) <= 4 and activation.is_cuda and activation.dim() == 2
+              and activation.dtype == torch.float32 and weight.dtype == torch.float32
+              and not torch.is_autocast_enabled() and weight.size(0) % 4 == 0)
+    if merged:
+        with torch.no_grad():
+            pos, neg = sc_extension_cuda.linear_generic_general_acc(
+                activation.data, weight.data, (prec_default, load_unit, load_wait_w), bit_length, LFSR_Length,
+                bin_config, gen_config, XNOR, MUX)
+            sc_value = _ops.sc_counts_to_float(pos, neg, bit_length)
+        if not (torch.is_grad_enabled() and (activation.requires_grad or weight.requires_grad)):
+            return sc_value
+        return Merged_Surrogate_Linear.apply(activation, weight, sc_value, or_n if or_n > 0 else 1)
     w_pos = weight.clamp(0, 100)
     w_neg = -(weight.clamp(-100, 0))
     lin_pos = F.linear(activation, w_pos)

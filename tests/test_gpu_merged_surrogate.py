@@ -166,3 +166,23 @@ def test_side_stream_overlap_changes_nothing(monkeypatch):
     assert torch.equal(ya, yb)
     _close(gxa, gxb, "grad x")   # MIOpen's gradient kernels accumulate with atomics: not bit-reproducible
     _close(gwa, gwb, "grad w")
+
+
+@pytest.mark.parametrize("forward", ["or_2", "or_1", "full_or"])
+def test_linear_merged_equals_two_gemms(forward, monkeypatch):
+    import sc_functional as uf
+    g = torch.Generator().manual_seed(31)
+    L = 64
+    x = torch.randint(0, L, (37, 200), generator=g).float() / L
+    w = torch.randint(-L + 1, L, (24, 200), generator=g).float() / L
+    gout = torch.randn(37, 24, generator=g).cuda()
+    res = []
+    for merged in ("1", "0"):
+        monkeypatch.setenv("REXSC_MERGED_SURROGATE", merged)
+        xt, wt = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+        y = uf.linear_generic_sc(xt, wt, bit_length=L, forward=forward, generator="lfsr", sync=1)
+        y.backward(gout)
+        res.append((y.detach().cpu(), xt.grad.cpu(), wt.grad.cpu()))
+    assert torch.equal(res[0][0], res[1][0])
+    _close(res[0][1], res[1][1], "grad x")
+    _close(res[0][2], res[1][2], "grad w")
