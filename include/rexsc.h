@@ -159,6 +159,11 @@ int rexsc_split_weight(const float *w, float *w2, size_t out_channels, size_t in
 int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t out_channels, size_t in_channels,
                             size_t taps, int dw2_channels_last, int w_channels_last, rexsc_stream_t stream);
 
+/* Fake quantisation y = clamp(round(x * 2^prec), -(2^prec - 1), 2^prec - 1) / 2^prec, round half to even,
+ * 0 <= prec <= 16: the mul / round / clamp / div passes of `quantize` (utils_functional.py:93-104, the
+ * forward of QuantizeGrad :117-123) in one.  n float32 elements of any dense layout; y may alias x. */
+int rexsc_quantize(const float *x, float *y, size_t n, int prec, rexsc_stream_t stream);
+
 /* Philox4x32-10 block function on the host (for known-answer tests of the generator). */
 void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
 

@@ -400,6 +400,17 @@ def merge_weight_grad(dw2, w):
     return dw
 
 
+def quantize(x, prec):
+    """clamp(round(x * 2^prec), +-(2^prec - 1)) / 2^prec in one pass, in x's layout."""
+    _require_cuda(x)
+    xd = _dense_f32(x)
+    y = torch.empty_like(xd)
+    with torch.cuda.device(xd.device):
+        rc = _lib.lib().rexsc_quantize(_ptr(xd), _ptr(y), xd.numel(), int(prec), _stream())
+        _lib.check(rc, "rexsc_quantize")
+    return y
+
+
 def calib_stats(a_bit, a_act, win_lo, win_hi):
     """count / sum / sum-of-squares of (a_bit - a_act) per window, float64 [n_win, 3] on device."""
     _require_cuda(a_bit, a_act)

@@ -430,6 +430,31 @@ __global__ __launch_bounds__(PW_THREADS) void merge_weight_grad_kernel(const flo
     dw[i] = gp - gn;
 }
 
+// Fake quantisation of activations and weights (utils_functional.py:93-104, prune = 0):
+// y = clamp(round_half_even(x * 2^prec), -(2^prec - 1), 2^prec - 1) / 2^prec; the scalings are exact.
+__device__ __forceinline__ float quantize_one(float x, float scale, float inv_scale, float lim)
+{
+    const float r = rintf(x * scale);
+    const float c = r != r ? r : fminf(fmaxf(r, 1.0f - scale), lim); // 1 - scale: +0 at prec 0, as torch's clamp bound
+    return c * inv_scale;
+}
+
+__global__ __launch_bounds__(PW_THREADS) void quantize_kernel(const float *__restrict__ x, float *__restrict__ y, size_t n,
+                                                             float scale, float inv_scale, float lim)
+{
+    const size_t nvec = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        const float4 v = reinterpret_cast<const float4 *>(x)[q];
+        float4 r;
+        r.x = quantize_one(v.x, scale, inv_scale, lim); r.y = quantize_one(v.y, scale, inv_scale, lim);
+        r.z = quantize_one(v.z, scale, inv_scale, lim); r.w = quantize_one(v.w, scale, inv_scale, lim);
+        reinterpret_cast<float4 *>(y)[q] = r;
+    }
+    const size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = quantize_one(x[i], scale, inv_scale, lim);
+}
+
 // Calibration statistics: per window k, count / sum / sum of squares of (a_bit - a_act) over
 // the elements with lo[k] <= a_act < hi[k].  Windows may overlap.
 constexpr int CAL_MAX_WIN = 64;
@@ -736,6 +761,21 @@ extern "C" int rexsc_merge_weight_grad(const float *dw2, const float *w, float *
     hipLaunchKernelGGL(merge_weight_grad_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS),
                        0, stream, dw2, w, dw, n, (unsigned)in_channels, (unsigned)taps, dw2_channels_last,
                        w_channels_last);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_quantize(const float *x, float *y, size_t n, int prec, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(prec >= 0 && prec <= 16, "prec must be 0..16 (got %d)", prec);
+    if (n == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(x && y, "null pointer");
+    const float scale = (float)(1u << prec);
+    const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("quantize", 8.0 * n, stream);
+    hipLaunchKernelGGL(quantize_kernel, dim3(grid), dim3(PW_THREADS), 0, stream, x, y, n, scale, 1.0f / scale,
+                       scale - 1.0f);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

@@ -182,3 +182,29 @@ def test_calibration_fit_matches_reference_python_on_gpu():
         return b.cpu().numpy(), s.cpu().numpy()
 
     check_calib_against_reference(fit)
+
+
+@pytest.mark.parametrize("prec", [0, 1, 5, 7, 8, 16])
+def test_fused_quantize_equals_the_four_torch_passes(prec):
+    """quantize (utils_functional.py:93-104) as one kernel: bit-equal to mul / round / clamp / div."""
+    import _ops
+    import sc_functional as uf
+    g = torch.Generator().manual_seed(prec)
+    s = 2.0 ** prec
+    x = torch.cat([
+        torch.randn(100003, generator=g) * 0.7,
+        (torch.arange(-40, 41).float() + 0.5) / s,            # ties: round half to even
+        torch.tensor([0.0, -0.0, 1.0, -1.0, 3.0, -3.0, 1 - 1 / s, 1e-30, -1e-30, 1e30, float("inf"), -float("inf"),
+                      float("nan")]),
+    ]).cuda()
+    want = (x * s).round().clamp(-s + 1, s - 1) / s
+    got = _ops.quantize(x, prec)
+    assert torch.equal(torch.nan_to_num(got, nan=9.0), torch.nan_to_num(want, nan=9.0))
+    assert torch.equal(torch.signbit(got), torch.signbit(want))
+    # through QuantizeGrad: same values, straight-through gradient, channels_last kept
+    x4 = torch.randn(2, 8, 5, 5, generator=g).cuda().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    y4 = uf.QuantizeGrad.apply(x4, prec)
+    assert y4.stride() == x4.stride()
+    assert torch.equal(y4, (x4.detach() * s).round().clamp(-s + 1, s - 1) / s)
+    y4.backward(torch.ones_like(y4))
+    assert torch.equal(x4.grad, torch.ones_like(x4))
