@@ -108,10 +108,13 @@ int rexsc_orn_backward(const float *grad_out, const float *x, float *grad_in, si
  * Replaces sc_extension_cuda.or_approx_n_forward_bias_std_both_acc / _backward_..._both_acc
  * (sc_cuda_pw.cu:863-927, 952-1011); scalar math of sc_cpu.hpp:264-404.
  * bias_coef / std_coef: 6 float32 coefficients each, device memory.
- * noise_out_pos / noise_out_neg: optional float32 [n] receiving the draws (NULL to skip). */
+ * noise_out_pos / noise_out_neg: optional float32 [n] receiving the draws (NULL to skip).
+ * offset_dev: optional device pointer to a uint64 added to `offset` when the kernel runs (NULL: none).
+ * A call recorded into a HIP graph has its host arguments frozen; a caller that advances *offset_dev on
+ * the stream after each call gets fresh noise on every replay. */
 int rexsc_orn_bias_std_both_forward(const float *x_pos, const float *x_neg, const float *bias_coef,
                                     const float *std_coef, float *y, size_t n, int or_n,
-                                    uint64_t seed, uint64_t offset,
+                                    uint64_t seed, uint64_t offset, const uint64_t *offset_dev,
                                     float *noise_out_pos, float *noise_out_neg, rexsc_stream_t stream);
 int rexsc_orn_bias_std_both_backward(const float *grad_out, const float *x_pos, const float *x_neg,
                                      const float *bias_coef, float *grad_pos, float *grad_neg, size_t n,
@@ -121,7 +124,7 @@ int rexsc_orn_bias_std_both_backward(const float *grad_out, const float *x_pos, 
  * binary16, as the reference's does. */
 int rexsc_orn_bias_std_forward_f16(const uint16_t *x_half, const float *bias_coef, const float *std_coef,
                                    uint16_t *y_half, size_t n, int or_n, uint64_t seed, uint64_t offset,
-                                   rexsc_stream_t stream);
+                                   const uint64_t *offset_dev, rexsc_stream_t stream);
 int rexsc_orn_bias_std_backward(const float *grad_out, const float *x, const float *bias_coef,
                                 float *grad_in, size_t n, int or_n, int half_input, rexsc_stream_t stream);
 
@@ -138,7 +141,7 @@ int rexsc_orn_pair_backward(const float *grad_out, const float *s2, float *g2, s
                             int or_n, int half_input, rexsc_stream_t stream);
 int rexsc_orn_bias_std_pair_forward(const float *s2, const float *bias_coef, const float *std_coef, float *y,
                                     size_t outer, size_t inner, int or_n, uint64_t seed, uint64_t offset,
-                                    rexsc_stream_t stream);
+                                    const uint64_t *offset_dev, rexsc_stream_t stream);
 int rexsc_orn_bias_std_pair_backward(const float *grad_out, const float *s2, const float *bias_coef, float *g2,
                                      size_t outer, size_t inner, int or_n, int half_input,
                                      rexsc_stream_t stream);

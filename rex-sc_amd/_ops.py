@@ -195,26 +195,36 @@ def orn_backward(grad_output, x, or_n, half_input=True):
     return gx
 
 
-_philox = {"seed": None, "offset": 0}
+_capture_counters = {}  # device index -> int64 [1] tensor: noise vectors consumed by captured calls
+_CAPTURE_SEED_SALT = 0x9E3779B97F4A7C15  # captured calls draw from a stream of their own
 
 
 def _next_philox(n_elems, device):
-    """(seed, offset) for the next noise draw, taken from the device's torch generator and advanced
-    past the 4-element vectors this call consumes -- the way the reference's kernels consume the
-    generator's Philox state (sc_cuda_pw.cu:870-877): torch.manual_seed restarts the stream.  While a
-    stream is being captured the generator may not be touched; a counter of this module stands in."""
+    """(seed, offset, counter) for the next noise draw.
+
+    Eagerly: seed and offset come from the device's torch generator, which is advanced past the
+    4-element vectors this call consumes -- the way the reference's kernels consume the generator's
+    Philox state (sc_cuda_pw.cu:870-877): torch.manual_seed restarts the stream; counter is None.
+    While a stream is being captured the host arguments are frozen into the graph, so the offset lives
+    in device memory instead: counter is an int64 tensor the kernel adds to its offset, and
+    _advance_philox() records its increment after the launch -- every replay draws new noise."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
     used = (n_elems + 3) // 4
+    gen = torch.cuda.default_generators[idx]
     if not torch.cuda.is_current_stream_capturing():
-        gen = torch.cuda.default_generators[device.index if device.index is not None else torch.cuda.current_device()]
+        if idx not in _capture_counters:  # allocated and zeroed outside any capture
+            _capture_counters[idx] = torch.zeros(1, dtype=torch.int64, device=device)
         seed, off = gen.initial_seed() & 0xFFFFFFFFFFFFFFFF, gen.get_offset()
         gen.set_offset(off + (used + 3) // 4 * 4)  # the generator keeps offsets in multiples of 4
-        return seed, off
-    seed = torch.initial_seed() & 0xFFFFFFFFFFFFFFFF
-    if _philox["seed"] != seed:
-        _philox["seed"], _philox["offset"] = seed, 0
-    off = _philox["offset"]
-    _philox["offset"] = off + used
-    return seed, off
+        return seed, off, None
+    if idx not in _capture_counters:
+        raise RuntimeError("noise kernels need one eager call on this device before they are captured")
+    return (torch.initial_seed() ^ _CAPTURE_SEED_SALT) & 0xFFFFFFFFFFFFFFFF, 0, _capture_counters[idx]
+
+
+def _advance_philox(counter, n_elems):
+    if counter is not None:
+        counter.add_((n_elems + 3) // 4)  # a kernel on the capturing stream: part of the graph
 
 
 def orn_bias_std_both_forward(x_pos, x_neg, bias_coef, std_coef, or_n, seed=None, offset=None, return_noise=False):
@@ -224,14 +234,17 @@ def orn_bias_std_both_forward(x_pos, x_neg, bias_coef, std_coef, or_n, seed=None
     b, s = _coef(bias_coef, xp.device), _coef(std_coef, xp.device)
     y = torch.empty_like(xp)
     n = xp.numel()
+    counter = None
     if seed is None:
-        seed, offset = _next_philox(n, xp.device)
+        seed, offset, counter = _next_philox(n, xp.device)
     np_ = torch.empty_like(xp) if return_noise else None
     nn_ = torch.empty_like(xp) if return_noise else None
     with torch.cuda.device(xp.device):
         rc = _lib.lib().rexsc_orn_bias_std_both_forward(_ptr(xp), _ptr(xn), _ptr(b), _ptr(s), _ptr(y), n, int(or_n),
-                                                        int(seed), int(offset), _ptr(np_), _ptr(nn_), _stream())
+                                                        int(seed), int(offset), _ptr(counter), _ptr(np_), _ptr(nn_),
+                                                        _stream())
         _lib.check(rc, "rexsc_orn_bias_std_both_forward")
+        _advance_philox(counter, n)
     return (y, np_, nn_) if return_noise else y
 
 
@@ -253,12 +266,14 @@ def orn_bias_std_forward_f16(x, bias_coef, std_coef, or_n, seed=None, offset=Non
     xh = x.detach().to(torch.float16).contiguous()
     b, s = _coef(bias_coef, xh.device), _coef(std_coef, xh.device)
     y = torch.empty_like(xh)
+    counter = None
     if seed is None:
-        seed, offset = _next_philox(xh.numel(), xh.device)
+        seed, offset, counter = _next_philox(xh.numel(), xh.device)
     with torch.cuda.device(xh.device):
         rc = _lib.lib().rexsc_orn_bias_std_forward_f16(_ptr(xh), _ptr(b), _ptr(s), _ptr(y), xh.numel(), int(or_n),
-                                                       int(seed), int(offset), _stream())
+                                                       int(seed), int(offset), _ptr(counter), _stream())
         _lib.check(rc, "rexsc_orn_bias_std_forward_f16")
+        _advance_philox(counter, xh.numel())
     return y
 
 
@@ -316,12 +331,14 @@ def orn_pair_backward(grad_output, s2, outer, inner, channels_last, or_n, half_i
 def orn_bias_std_pair_forward(s2, outer, inner, channels_last, bias_coef, std_coef, or_n, seed=None, offset=None):
     b, s = _coef(bias_coef, s2.device), _coef(std_coef, s2.device)
     y = _pair_result_like(s2, channels_last)
+    counter = None
     if seed is None:
-        seed, offset = _next_philox(y.numel(), y.device)
+        seed, offset, counter = _next_philox(y.numel(), y.device)
     with torch.cuda.device(s2.device):
         rc = _lib.lib().rexsc_orn_bias_std_pair_forward(_ptr(s2), _ptr(b), _ptr(s), _ptr(y), outer, inner, int(or_n),
-                                                        int(seed), int(offset), _stream())
+                                                        int(seed), int(offset), _ptr(counter), _stream())
         _lib.check(rc, "rexsc_orn_bias_std_pair_forward")
+        _advance_philox(counter, y.numel())
     return y
 
 

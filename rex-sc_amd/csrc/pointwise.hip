@@ -177,9 +177,10 @@ __global__ __launch_bounds__(PW_THREADS) void orn_backward_kernel(const float *_
 template <int N>
 __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_both_forward_kernel(
     const float *__restrict__ xp, const float *__restrict__ xn, const float *__restrict__ bc, const float *__restrict__ sc,
-    float *__restrict__ y, size_t n, uint64_t seed, uint64_t offset, float *__restrict__ noise_p,
-    float *__restrict__ noise_n)
+    float *__restrict__ y, size_t n, uint64_t seed, uint64_t offset, const uint64_t *__restrict__ offset_dev,
+    float *__restrict__ noise_p, float *__restrict__ noise_n)
 {
+    if (offset_dev) offset += *offset_dev; // wave-uniform: a scalar load
     const Coef6 b = load_coef(bc), s = load_coef(sc);
     const size_t nvec = (n + 3) / 4; // the tail vector is handled element-wise below
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -249,8 +250,10 @@ __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_forward_f16_kernel(co
                                                                               const float *__restrict__ bc,
                                                                               const float *__restrict__ sc,
                                                                               __half *__restrict__ y, size_t n,
-                                                                              uint64_t seed, uint64_t offset)
+                                                                              uint64_t seed, uint64_t offset,
+                                                                              const uint64_t *__restrict__ offset_dev)
 {
+    if (offset_dev) offset += *offset_dev;
     const Coef6 b = load_coef(bc), s = load_coef(sc);
     const size_t nvec = (n + 3) / 4;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -321,8 +324,9 @@ __global__ __launch_bounds__(PW_THREADS) void orn_pair_backward_kernel(const flo
 template <int N>
 __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_pair_forward_kernel(
     const float *__restrict__ s2, const float *__restrict__ bc, const float *__restrict__ sc, float *__restrict__ y,
-    size_t nvec, unsigned inner4, uint64_t seed, uint64_t offset)
+    size_t nvec, unsigned inner4, uint64_t seed, uint64_t offset, const uint64_t *__restrict__ offset_dev)
 {
+    if (offset_dev) offset += *offset_dev;
     const Coef6 b = load_coef(bc), s = load_coef(sc);
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
@@ -570,7 +574,8 @@ extern "C" int rexsc_orn_backward(const float *g, const float *x, float *gx, siz
 
 extern "C" int rexsc_orn_bias_std_both_forward(const float *xp, const float *xn, const float *bias_coef,
                                                const float *std_coef, float *y, size_t n, int or_n, uint64_t seed,
-                                               uint64_t offset, float *noise_p, float *noise_n, rexsc_stream_t stream_)
+                                               uint64_t offset, const uint64_t *offset_dev, float *noise_p,
+                                               float *noise_n, rexsc_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
@@ -579,8 +584,8 @@ extern "C" int rexsc_orn_bias_std_both_forward(const float *xp, const float *xn,
     const int grid = pw_grid((n + 3) / 4);
     ProfScope prof("orn_bias_std_both_forward", (12.0 + (noise_p ? 4.0 : 0.0) + (noise_n ? 4.0 : 0.0)) * n, stream);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_both_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
-                                               stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, noise_p,
-                                               noise_n));
+                                               stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, offset_dev,
+                                               noise_p, noise_n));
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
@@ -603,7 +608,7 @@ extern "C" int rexsc_orn_bias_std_both_backward(const float *g, const float *xp,
 
 extern "C" int rexsc_orn_bias_std_forward_f16(const uint16_t *x_half, const float *bias_coef, const float *std_coef,
                                               uint16_t *y_half, size_t n, int or_n, uint64_t seed, uint64_t offset,
-                                              rexsc_stream_t stream_)
+                                              const uint64_t *offset_dev, rexsc_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
@@ -612,7 +617,7 @@ extern "C" int rexsc_orn_bias_std_forward_f16(const uint16_t *x_half, const floa
     const int grid = pw_grid((n + 3) / 4);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_forward_f16_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
                                                stream, reinterpret_cast<const __half *>(x_half), bias_coef, std_coef,
-                                               reinterpret_cast<__half *>(y_half), n, seed, offset));
+                                               reinterpret_cast<__half *>(y_half), n, seed, offset, offset_dev));
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
@@ -685,7 +690,7 @@ extern "C" int rexsc_orn_pair_backward(const float *g, const float *s2, float *g
 
 extern "C" int rexsc_orn_bias_std_pair_forward(const float *s2, const float *bias_coef, const float *std_coef, float *y,
                                                size_t outer, size_t inner, int or_n, uint64_t seed, uint64_t offset,
-                                               rexsc_stream_t stream_)
+                                               const uint64_t *offset_dev, rexsc_stream_t stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
@@ -697,7 +702,7 @@ extern "C" int rexsc_orn_bias_std_pair_forward(const float *s2, const float *bia
     ProfScope prof("orn_bias_std_pair_forward", 12.0 * outer * inner, stream);
     REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_pair_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
                                                stream, s2, bias_coef, std_coef, y, nvec, (unsigned)(inner / 4), seed,
-                                               offset));
+                                               offset, offset_dev));
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

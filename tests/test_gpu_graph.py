@@ -94,3 +94,28 @@ def test_fixed_conv_and_pointwise_graph():
 
     g, out = _capture(fn)
     _check_replays(g, out, fn, refill)
+
+
+def test_error_injection_draws_new_noise_on_every_replay():
+    """A captured noise kernel has its host arguments frozen; its offset lives in device memory and
+    is advanced inside the graph, so replays differ from each other the way eager calls do."""
+    import sc_extension_cuda
+    print("graph noise", flush=True)
+    x = torch.rand(20000, device="cuda")
+    coef0 = torch.zeros(6, device="cuda")
+    std = torch.tensor([0.25, 0, 0, 0, 0, 0], device="cuda")
+    fn = lambda: sc_extension_cuda.or_approx_n_forward_bias_std_both_acc(x, x, coef0, std, 2)
+    g, out = _capture(fn)
+    seen = []
+    for r in range(4):
+        g.replay()
+        torch.cuda.synchronize()
+        seen.append(out.clone())
+        _ = fn()                      # eager work between the replays
+        torch.cuda.synchronize()
+    for i in range(4):
+        for j in range(i):
+            d = (seen[i] - seen[j]) / 0.25
+            assert not torch.equal(seen[i], seen[j])
+            assert abs(float(d.var()) - 4.0) < 0.3   # four independent N(0,1) draws per element
+        assert abs(float(seen[i].mean())) < 0.02     # same operand on both polarities: zero-mean output
