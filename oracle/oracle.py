@@ -9,10 +9,17 @@ with numpy arrays in place of tensors, so a parity test reads like a call of the
 compute_bias_std_coef restates utils_functional.py:900-949 in numpy (float64 statistics
 are NOT used: the reference works in float32 tensors, and so does this).
 
-Pinning: the conv / linear / fixed-conv functions against tests/golden/ref_cpu_ext.npz (written by
-the reference's compiled CPU extension), compute_bias_std_coef against tests/golden/ref_calib.npz
+Pinning: the conv / linear / fixed-conv functions against tests/golden/ref_cpu_ext.npz (hand-picked
+cases) and ref_cpu_ext_random.npz (96 seeded random configurations), both written by the
+reference's compiled CPU extension; compute_bias_std_coef against tests/golden/ref_calib.npz
 (written by the reference's own Python function); the scalar float functions (OR-n, bias/noise,
 quantise) against closed forms in tests/test_oracle_invariants.py.
+
+Parity unpinned: the linear op with an 8-bit LFSR (256-bit streams or lfsr_length 8).  The
+reference has no defined result there: built with AVX-512 it calls an uninitialised step-function
+pointer (sc_matmul.cpp:48-70 has no case for 8 bits) and faults; built without AVX-512 its linear
+op returns different numbers on repeated calls with the same operands.  The oracle continues the
+7-bit rules with the 8-bit step function that the conv op is pinned on.
 """
 import ctypes
 import os

@@ -9,8 +9,30 @@ import pytest
 import oracle as orc
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-_data = np.load(os.path.join(ROOT, "tests", "golden", "ref_cpu_ext.npz"), allow_pickle=False)
-_meta = json.loads(bytes(_data["meta"]).decode())
+
+
+class _Golden:
+    """The two fixtures written by the reference's compiled CPU extension: hand-picked cases
+    (make_golden.py) and seeded random configurations (make_golden_random.py), as one key space."""
+
+    def __init__(self):
+        self.files = [np.load(os.path.join(ROOT, "tests", "golden", f), allow_pickle=False)
+                      for f in ("ref_cpu_ext.npz", "ref_cpu_ext_random.npz")]
+        self.meta = {"conv": [], "linear": [], "fixed": []}
+        for f in self.files:
+            m = json.loads(bytes(f["meta"]).decode())
+            for kind in self.meta:
+                self.meta[kind] += m[kind]
+
+    def __getitem__(self, key):
+        for f in self.files:
+            if key in f.files:
+                return f[key]
+        raise KeyError(key)
+
+
+_data = _Golden()
+_meta = _data.meta
 
 
 @pytest.mark.parametrize("case", _meta["conv"], ids=lambda c: c["name"])
