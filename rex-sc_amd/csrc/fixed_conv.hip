@@ -171,14 +171,14 @@ struct Fixed8Params {
     float P2;
 };
 
-__global__ __launch_bounds__(256) void fixed_pack_act16_kernel(const float *__restrict__ x, int8_t *__restrict__ xq16,
-                                                               Fixed8Params p)
+__device__ __forceinline__ void fixed_pack_act16(const float *__restrict__ x, int8_t *__restrict__ xq16,
+                                                 const Fixed8Params &p, unsigned bid)
 {
     // one thread per (n, cb, yp, xp): 16 channels -> 16 bytes.  A block stays inside one (n, cb)
     // plane (blocks_per_plane blocks each), so the per-thread index arithmetic is one 32-bit division.
     const unsigned plane = (unsigned)p.Hp * p.Wp;
     const unsigned blocks_per_plane = (plane + 255) / 256;
-    const unsigned ncb = blockIdx.x / blocks_per_plane, pblk = blockIdx.x - ncb * blocks_per_plane;
+    const unsigned ncb = bid / blocks_per_plane, pblk = bid - ncb * blocks_per_plane;
     const unsigned n = ncb / (unsigned)p.CB, cb = ncb - n * (unsigned)p.CB;
     const long in_plane = (long)p.H * p.W;
     {
@@ -198,14 +198,15 @@ __global__ __launch_bounds__(256) void fixed_pack_act16_kernel(const float *__re
     }
 }
 
-__global__ __launch_bounds__(256) void fixed_pack_w16_kernel(const float *__restrict__ w, int8_t *__restrict__ wq16,
-                                                             int8_t *__restrict__ wp16, Fixed8Params p)
+__device__ __forceinline__ void fixed_pack_w16(const float *__restrict__ w, int8_t *__restrict__ wq16,
+                                               int8_t *__restrict__ wp16, const Fixed8Params &p, unsigned bid,
+                                               unsigned n_blocks)
 {
     // one thread per (cb, o, tap), tap fastest: the threads of one (cb, o) read one contiguous run of
     // the OIHW weights (16 channels x KH*KW taps) between them; each writes its 16-byte entries.
     const unsigned taps = (unsigned)(p.KH * p.KW);
     const unsigned total = (unsigned)p.CB * p.O_pad * taps;
-    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+    for (unsigned i = bid * 256 + threadIdx.x; i < total; i += n_blocks * 256) {
         const unsigned tap = i % taps, co = i / taps;
         const unsigned o = co % (unsigned)p.O_pad, cb = co / (unsigned)p.O_pad;
         uint32_t vals[4] = {0, 0, 0, 0}, pars[4] = {0, 0, 0, 0};
@@ -228,10 +229,29 @@ __global__ __launch_bounds__(256) void fixed_pack_w16_kernel(const float *__rest
     }
 }
 
-__global__ void fixed_zero_kernel(int32_t *__restrict__ p, size_t n)
+// One launch prepares everything the MFMA kernel needs: blocks [0, act_blocks) pack the activations,
+// the next w_blocks pack the weights, the last zero_blocks clear the output when the reduction is split
+// over blocks that add their parts atomically.  (Three launches of this size cost more in launch
+// latency than in work.)
+__global__ __launch_bounds__(256) void fixed_prepare_kernel(const float *__restrict__ x, int8_t *__restrict__ xq16,
+                                                            const float *__restrict__ w, int8_t *__restrict__ wq16,
+                                                            int8_t *__restrict__ wp16, int32_t *__restrict__ out,
+                                                            size_t n_out, Fixed8Params p, unsigned act_blocks,
+                                                            unsigned w_blocks, unsigned zero_blocks)
 {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = 0;
+    unsigned bid = blockIdx.x;
+    if (bid < act_blocks) { fixed_pack_act16(x, xq16, p, bid); return; }
+    bid -= act_blocks;
+    if (bid < w_blocks) { fixed_pack_w16(w, wq16, wp16, p, bid, w_blocks); return; }
+    bid -= w_blocks;
+    if ((reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+        uint4 *o4 = reinterpret_cast<uint4 *>(out);
+        const size_t n4 = n_out / 4;
+        for (size_t i = (size_t)bid * 256 + threadIdx.x; i < n4; i += (size_t)zero_blocks * 256) o4[i] = make_uint4(0, 0, 0, 0);
+        if (bid == 0 && threadIdx.x < (n_out & 3)) out[n4 * 4 + threadIdx.x] = 0;
+    } else {
+        for (size_t i = (size_t)bid * 256 + threadIdx.x; i < n_out; i += (size_t)zero_blocks * 256) out[i] = 0;
+    }
 }
 
 // A block of 4 waves computes a 64 (channels) x 256 (pixels) tile over its share of the channel-block
@@ -364,6 +384,190 @@ __global__ __launch_bounds__(256) void fixed_mfma_kernel(const int8_t *__restric
     }
 }
 
+// Persistent variant for KH x KW known at compile time: a block walks over its work items
+// (256-pixel group, 64-channel tile, share of the channel-block pairs) and over the pairs of each item
+// with the weights double-buffered in LDS: the 16-byte entries of the next pair are requested from L2
+// before the MFMAs of the current pair are issued and written to the other buffer after them, so a
+// pair costs one barrier and no exposed staging latency.  A buffer that already holds the pair it is
+// asked for is left alone: with one or two pairs and one channel tile (C <= 64, O <= 64) the weights
+// stay resident for the whole launch.
+template <int KH, int KW, int PB>
+__global__ __launch_bounds__(256) void fixed_mfma_db_kernel(const int8_t *__restrict__ xq16, const int8_t *__restrict__ wq16,
+                                                            const int8_t *__restrict__ wp16, int32_t *__restrict__ out,
+                                                            Fixed8Params p, int n_items)
+{
+    constexpr int TAPS = KH * KW;
+    constexpr int ENT = 2 * TAPS * 2 * FT; // 16-byte entries of one pair: [h][tap][val/par][o 0..63]
+    static_assert(ENT % 256 == 0, "entries must divide among the threads");
+    constexpr int EPT = ENT / 256;
+    constexpr int WPX = 32 * PB;
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_raw[];
+    v4i *s_w = reinterpret_cast<v4i *>(s_raw); // two buffers of ENT entries
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31, h = lane >> 5;
+    const int o_tiles = p.O_pad / FT;
+    const long plane = (long)p.Hp * p.Wp;
+    const int HoWo = p.Ho * p.Wo;
+    const v4i *xb = reinterpret_cast<const v4i *>(xq16);
+    const v4i *wb = reinterpret_cast<const v4i *>(wq16);
+    const v4i *wpb = reinterpret_cast<const v4i *>(wp16);
+    const long wkk = (long)TAPS * p.O_pad;
+    const int pairs = p.CB / 2;
+    const int per = (pairs + p.ksplit - 1) / p.ksplit;
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+
+    // where thread t's e-th entry of pair (otile, cbp) comes from
+    auto entry_src = [&](int e, int otile, int cbp, bool &is_par) -> long {
+        const int o = e % FT, vp = (e / FT) % 2, tap = (e / (2 * FT)) % TAPS, hh = e / (2 * FT * TAPS);
+        is_par = vp != 0;
+        return (long)(2 * cbp + hh) * wkk + (long)tap * p.O_pad + otile * FT + o;
+    };
+
+    int held0 = -1, held1 = -1; // pair id (otile * pairs + cbp) in each buffer; block-uniform
+    int step = 0;
+    v4i stage[EPT];
+
+    for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
+        int t = item;
+        const int ks = t % p.ksplit; t /= p.ksplit;
+        const int otile = t % o_tiles;
+        const long mtile = (long)(t / o_tiles) * 4 + wave;
+        const int cbp_begin = ks * per, cbp_end = min(pairs, cbp_begin + per);
+        // the next item's first pair, for the prefetch across the item boundary
+        int n_otile = -1, n_cbp = -1;
+        if (item + (int)gridDim.x < n_items) {
+            int u = item + gridDim.x;
+            const int nks = u % p.ksplit; u /= p.ksplit;
+            n_otile = u % o_tiles; n_cbp = nks * per;
+            if (n_cbp >= pairs) n_otile = -1;
+        }
+
+        long xoff[PB];
+        int mm[PB];
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            const long m = mtile * WPX + pb * 32 + j;
+            mm[pb] = (int)(m < p.M ? m : p.M - 1);
+            const int n = mm[pb] / HoWo, r = mm[pb] - n * HoWo;
+            const int yo = r / p.Wo, xo = r - yo * p.Wo;
+            xoff[pb] = (long)n * p.CB * plane + (long)(yo * p.s0) * p.Wp + xo * p.s1;
+            if (m >= p.M) mm[pb] = -1;
+        }
+        v16i acc[2][PB];
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < PB; b++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
+
+        v4i bc[PB][KW], bn[PB][KW];
+        if (cbp_begin < cbp_end) {
+            const v4i *xc = xb + (long)(2 * cbp_begin + h) * plane;
+#pragma unroll
+            for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++) bc[pb][kx] = xc[xoff[pb] + kx];
+        }
+        for (int cbp = cbp_begin; cbp < cbp_end; cbp++, step++) {
+            const int buf = step & 1;
+            const int id = otile * pairs + cbp;
+            if ((buf ? held1 : held0) != id) {
+                // not prefetched (first step of the block): stage it now
+#pragma unroll
+                for (int e = 0; e < EPT; e++) {
+                    bool par;
+                    const long src = entry_src(threadIdx.x + e * 256, otile, cbp, par);
+                    stage[e] = par ? wpb[src] : wb[src];
+                }
+#pragma unroll
+                for (int e = 0; e < EPT; e++) s_w[buf * ENT + threadIdx.x + e * 256] = stage[e];
+                if (buf) held1 = id; else held0 = id;
+                __syncthreads();
+            }
+            // the pair of the next step, into the other buffer
+            int p_otile = otile, p_cbp = cbp + 1;
+            if (p_cbp >= cbp_end) { p_otile = n_otile; p_cbp = n_cbp; }
+            const int nid = p_otile >= 0 ? p_otile * pairs + p_cbp : -1;
+            const bool prefetch = nid >= 0 && (buf ? held0 : held1) != nid;
+            if (prefetch) {
+#pragma unroll
+                for (int e = 0; e < EPT; e++) {
+                    bool par;
+                    const long src = entry_src(threadIdx.x + e * 256, p_otile, p_cbp, par);
+                    stage[e] = par ? wpb[src] : wb[src];
+                }
+            }
+            const v4i *sw = s_w + buf * ENT + (long)h * TAPS * 2 * FT + j;
+#pragma unroll
+            for (int ky = 0; ky < KH; ky++) {
+                {
+                    int cn = cbp, kn = ky + 1;
+                    if (kn == KH) { kn = 0; cn = cbp + 1; }
+                    if (cn >= cbp_end) { cn = cbp; kn = ky; }
+                    const v4i *xn = xb + (long)(2 * cn + h) * plane + (long)kn * p.Wp;
+#pragma unroll
+                    for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                        for (int kx = 0; kx < KW; kx++) bn[pb][kx] = xn[xoff[pb] + kx];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++) {
+                    const v4i *wt = sw + (ky * KW + kx) * 2 * FT;
+                    const v4i a0 = wt[0], a1 = wt[32], q0 = wt[FT], q1 = wt[FT + 32];
+#pragma unroll
+                    for (int pb = 0; pb < PB; pb++) {
+                        acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bc[pb][kx], acc[0][pb], 0, 0, 0);
+                        acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bc[pb][kx], acc[1][pb], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int pb = 0; pb < PB; pb++) {
+                        const v4i par = bc[pb][kx] & ones;
+                        acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, par, acc[0][pb], 0, 0, 0);
+                        acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, par, acc[1][pb], 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+                    for (int kx = 0; kx < KW; kx++) bc[pb][kx] = bn[pb][kx];
+            }
+            if (prefetch) {
+#pragma unroll
+                for (int e = 0; e < EPT; e++) s_w[(buf ^ 1) * ENT + threadIdx.x + e * 256] = stage[e];
+                if (buf) held0 = nid; else held1 = nid;
+            }
+            // everyone is done reading this step's buffer (it is the next prefetch target) and the
+            // other buffer is complete
+            __syncthreads();
+        }
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++) {
+            if (mm[pb] < 0) continue;
+            const int n = mm[pb] / HoWo, r0 = mm[pb] - n * HoWo;
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int o = otile * FT + a * 32 + 8 * (r / 4) + 4 * h + (r % 4);
+                    if (o >= p.O) continue;
+                    int32_t *dst = out + ((long)n * p.O + o) * HoWo + r0;
+                    if (p.ksplit == 1) *dst = acc[a][pb][r];
+                    else atomicAdd(dst, acc[a][pb][r]);
+                }
+        }
+    }
+}
+
+static int tune_flag(const char *name, int dflt)
+{
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) : dflt;
+}
+
 // The MFMA path is exact only where the per-product saturating add is provably inert.
 static bool fixed_use_mfma(const FixedParams &p)
 {
@@ -446,7 +650,15 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         q.ksplit = 1;
         // (the atomic epilogue of a split costs about as much as the MFMA work of a wave: split only
         // while the launch has fewer wave tiles than about one per SIMD)
-        while (tiles * q.ksplit < 1024 && q.ksplit * 2 <= q.CB / 2) q.ksplit *= 2;
+        const bool db_shape = q.KH == 3 && q.KW == 3 && pb == 2 && tune_flag("REXSC_TUNE_FIXED_DB", 1);
+        if (db_shape) {
+            // persistent kernel (staging overlapped, long blocks): split only while the work items would
+            // not even give every CU one block
+            const long items = (((long)ceil_div(q.M, wpx) + 3) / 4) * (q.O_pad / FT);
+            while (items * q.ksplit * 2 <= 256 && q.ksplit * 2 <= q.CB / 2) q.ksplit *= 2;
+        } else {
+            while (tiles * q.ksplit < 1024 && q.ksplit * 2 <= q.CB / 2) q.ksplit *= 2;
+        }
         if (getenv("REXSC_TUNE_FIXED_KSPLIT")) {
             q.ksplit = atoi(getenv("REXSC_TUNE_FIXED_KSPLIT"));
             if (q.ksplit < 1) q.ksplit = 1;
@@ -462,17 +674,38 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
             ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 16.0 * q.N * q.CB * q.Hp * q.Wp, stream);
             const long pack_blocks = (((long)q.Hp * q.Wp + 255) / 256) * q.N * q.CB;
             REXSC_CHECK_ARG(pack_blocks < (1L << 31) && (long)q.CB * q.O_pad * q.KH * q.KW < (1L << 31), "fixed conv2d: problem too large");
-            hipLaunchKernelGGL(fixed_pack_act16_kernel, dim3((unsigned)pack_blocks), dim3(256), 0, stream, x, xq16, q);
-            hipLaunchKernelGGL(fixed_pack_w16_kernel, dim3(gridf((long)q.CB * q.O_pad * q.KH * q.KW)), dim3(256), 0, stream, w, wq16,
-                               wp16, q);
-            if (q.ksplit > 1)
-                hipLaunchKernelGGL(fixed_zero_kernel, dim3(gridf((long)nout / 4 + 1)), dim3(256), 0, stream, out, nout);
+            const unsigned w_blocks = (unsigned)gridf((long)q.CB * q.O_pad * q.KH * q.KW);
+            unsigned zero_blocks = 0;
+            if (q.ksplit > 1) {
+                zero_blocks = (unsigned)gridf((long)nout / 4 + 1);
+                if (zero_blocks > 2048) zero_blocks = 2048;
+            }
+            REXSC_CHECK_ARG(pack_blocks + w_blocks + zero_blocks < (1L << 31), "fixed conv2d: problem too large");
+            hipLaunchKernelGGL(fixed_prepare_kernel, dim3((unsigned)pack_blocks + w_blocks + zero_blocks), dim3(256), 0,
+                               stream, x, xq16, w, wq16, wp16, out, nout, q, (unsigned)pack_blocks, w_blocks, zero_blocks);
         }
         REXSC_CHECK_HIP(hipGetLastError());
         const long m_groups = ((long)ceil_div(q.M, wpx) + 3) / 4;
         const unsigned grid = (unsigned)(m_groups * (q.O_pad / FT) * q.ksplit);
         const size_t lds = (size_t)2 * q.KH * q.KW * 2 * FT * 16;
         ProfScope prof("fixed_conv_mfma", io_bytes, stream);
+        if (db_shape) {
+            static bool attr_set[64] = {}; // per device: the kernel needs more than the default 64 KB of LDS
+            const size_t lds2 = 2 * lds;
+            int dev = 0;
+            REXSC_CHECK_HIP(hipGetDevice(&dev));
+            if (dev < 0 || dev >= 64 || !attr_set[dev]) {
+                REXSC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&fixed_mfma_db_kernel<3, 3, 2>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
+                if (dev >= 0 && dev < 64) attr_set[dev] = true;
+            }
+            const long n_items = (long)grid;
+            const unsigned pgrid = (unsigned)(n_items < 512 ? n_items : 512); // two blocks per CU stay resident
+            hipLaunchKernelGGL((fixed_mfma_db_kernel<3, 3, 2>), dim3(pgrid), dim3(256), lds2, stream, xq16, wq16, wp16, out,
+                               q, (int)n_items);
+            REXSC_CHECK_HIP(hipGetLastError());
+            return REXSC_OK;
+        }
         switch (q.KW) {
         case 1:
             if (pb == 1) hipLaunchKernelGGL((fixed_mfma_kernel<1, 1>), dim3(grid), dim3(256), lds, stream, xq16, wq16, wp16, out, q);
