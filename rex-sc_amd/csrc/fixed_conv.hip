@@ -426,7 +426,6 @@ __global__ __launch_bounds__(256) void fixed_mfma_db_kernel(const int8_t *__rest
 
     int held0 = -1, held1 = -1; // pair id (otile * pairs + cbp) in each buffer; block-uniform
     int step = 0;
-    v4i stage[EPT];
 
     for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
         int t = item;
@@ -462,19 +461,28 @@ __global__ __launch_bounds__(256) void fixed_mfma_db_kernel(const int8_t *__rest
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
 
-        v4i bc[PB][KW], bn[PB][KW];
-        if (cbp_begin < cbp_end) {
-            const v4i *xc = xb + (long)(2 * cbp_begin + h) * plane;
+        // Activation rows (one per (pair, ky)) run through a ring of KH register sets: row r lives in set
+        // r % KH = ky, and the row two steps ahead is requested before the MFMAs of the current row, so a
+        // load has two rows of MFMAs (and the other wave's) to arrive.
+        static_assert(KH >= 3, "the ring holds the current row and two rows in flight");
+        v4i rows[KH][PB][KW];
+        const int n_rows = (cbp_end - cbp_begin) * KH;
+        auto load_row = [&](int r, v4i (&dst)[PB][KW]) {
+            r = r < n_rows ? r : n_rows - 1; // past the end: re-read the last row (harmless)
+            const int cb = cbp_begin + r / KH, ky = r - (r / KH) * KH;
+            const v4i *xr = xb + (long)(2 * cb + h) * plane + (long)ky * p.Wp;
 #pragma unroll
             for (int pb = 0; pb < PB; pb++)
 #pragma unroll
-                for (int kx = 0; kx < KW; kx++) bc[pb][kx] = xc[xoff[pb] + kx];
-        }
+                for (int kx = 0; kx < KW; kx++) dst[pb][kx] = xr[xoff[pb] + kx];
+        };
+        if (n_rows > 0) { load_row(0, rows[0]); load_row(1, rows[1]); }
         for (int cbp = cbp_begin; cbp < cbp_end; cbp++, step++) {
             const int buf = step & 1;
             const int id = otile * pairs + cbp;
             if ((buf ? held1 : held0) != id) {
                 // not prefetched (first step of the block): stage it now
+                v4i stage[EPT];
 #pragma unroll
                 for (int e = 0; e < EPT; e++) {
                     bool par;
@@ -486,32 +494,28 @@ __global__ __launch_bounds__(256) void fixed_mfma_db_kernel(const int8_t *__rest
                 if (buf) held1 = id; else held0 = id;
                 __syncthreads();
             }
-            // the pair of the next step, into the other buffer
+            // the pair of the next step goes into the other buffer, a third of it per kernel row
             int p_otile = otile, p_cbp = cbp + 1;
             if (p_cbp >= cbp_end) { p_otile = n_otile; p_cbp = n_cbp; }
             const int nid = p_otile >= 0 ? p_otile * pairs + p_cbp : -1;
             const bool prefetch = nid >= 0 && (buf ? held0 : held1) != nid;
-            if (prefetch) {
-#pragma unroll
-                for (int e = 0; e < EPT; e++) {
-                    bool par;
-                    const long src = entry_src(threadIdx.x + e * 256, p_otile, p_cbp, par);
-                    stage[e] = par ? wpb[src] : wb[src];
-                }
-            }
+            constexpr int EPR = (EPT + KH - 1) / KH; // entries per thread and row
             const v4i *sw = s_w + buf * ENT + (long)h * TAPS * 2 * FT + j;
+            const int r_base = (cbp - cbp_begin) * KH;
 #pragma unroll
             for (int ky = 0; ky < KH; ky++) {
-                {
-                    int cn = cbp, kn = ky + 1;
-                    if (kn == KH) { kn = 0; cn = cbp + 1; }
-                    if (cn >= cbp_end) { cn = cbp; kn = ky; }
-                    const v4i *xn = xb + (long)(2 * cn + h) * plane + (long)kn * p.Wp;
+                v4i stage[EPR];
+                if (prefetch) {
 #pragma unroll
-                    for (int pb = 0; pb < PB; pb++)
-#pragma unroll
-                        for (int kx = 0; kx < KW; kx++) bn[pb][kx] = xn[xoff[pb] + kx];
+                    for (int e = 0; e < EPR; e++) {
+                        if (ky * EPR + e < EPT) {
+                            bool par;
+                            const long src = entry_src(threadIdx.x + (ky * EPR + e) * 256, p_otile, p_cbp, par);
+                            stage[e] = par ? wpb[src] : wb[src];
+                        }
+                    }
                 }
+                load_row(r_base + ky + 2, rows[(ky + 2) % KH]);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kx = 0; kx < KW; kx++) {
@@ -519,27 +523,24 @@ __global__ __launch_bounds__(256) void fixed_mfma_db_kernel(const int8_t *__rest
                     const v4i a0 = wt[0], a1 = wt[32], q0 = wt[FT], q1 = wt[FT + 32];
 #pragma unroll
                     for (int pb = 0; pb < PB; pb++) {
-                        acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, bc[pb][kx], acc[0][pb], 0, 0, 0);
-                        acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, bc[pb][kx], acc[1][pb], 0, 0, 0);
+                        acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, rows[ky][pb][kx], acc[0][pb], 0, 0, 0);
+                        acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, rows[ky][pb][kx], acc[1][pb], 0, 0, 0);
                     }
 #pragma unroll
                     for (int pb = 0; pb < PB; pb++) {
-                        const v4i par = bc[pb][kx] & ones;
+                        const v4i par = rows[ky][pb][kx] & ones;
                         acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, par, acc[0][pb], 0, 0, 0);
                         acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, par, acc[1][pb], 0, 0, 0);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                if (prefetch) {
 #pragma unroll
-                for (int pb = 0; pb < PB; pb++)
-#pragma unroll
-                    for (int kx = 0; kx < KW; kx++) bc[pb][kx] = bn[pb][kx];
+                    for (int e = 0; e < EPR; e++)
+                        if (ky * EPR + e < EPT) s_w[(buf ^ 1) * ENT + threadIdx.x + (ky * EPR + e) * 256] = stage[e];
+                }
             }
-            if (prefetch) {
-#pragma unroll
-                for (int e = 0; e < EPT; e++) s_w[(buf ^ 1) * ENT + threadIdx.x + e * 256] = stage[e];
-                if (buf) held0 = nid; else held1 = nid;
-            }
+            if (prefetch) { if (buf) held0 = nid; else held1 = nid; }
             // everyone is done reading this step's buffer (it is the next prefetch target) and the
             // other buffer is complete
             __syncthreads();
