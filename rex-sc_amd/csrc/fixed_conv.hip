@@ -645,13 +645,15 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         q.CB = (int)align_up((size_t)ceil_div(p.C, 16), 2); q.M = p.N * p.Ho * p.Wo; q.P2 = p.P2;
         // split the channel-block pairs over waves until the launch has a few thousand of them
         int pb = 2;
+        const bool db_shape = q.KH == 3 && q.KW == 3 && tune_flag("REXSC_TUNE_FIXED_DB", 1);
+        // persistent kernel: 32-pixel waves when 64-pixel waves would leave SIMDs without any
+        if (db_shape && (long)ceil_div(q.M, 64) * (q.O_pad / FT) < 1024) pb = 1;
         if (getenv("REXSC_TUNE_FIXED_PB")) pb = atoi(getenv("REXSC_TUNE_FIXED_PB")) == 1 ? 1 : 2;
         const int wpx = 32 * pb;
         const long tiles = (long)ceil_div(q.M, wpx) * (q.O_pad / FT);
         q.ksplit = 1;
         // (the atomic epilogue of a split costs about as much as the MFMA work of a wave: split only
         // while the launch has fewer wave tiles than about one per SIMD)
-        const bool db_shape = q.KH == 3 && q.KW == 3 && pb == 2 && tune_flag("REXSC_TUNE_FIXED_DB", 1);
         if (db_shape) {
             // persistent kernel (staging overlapped, long blocks): split only while the work items would
             // not even give every CU one block
@@ -698,12 +700,18 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
             if (dev < 0 || dev >= 64 || !attr_set[dev]) {
                 REXSC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&fixed_mfma_db_kernel<3, 3, 2>),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
+                REXSC_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&fixed_mfma_db_kernel<3, 3, 1>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
                 if (dev >= 0 && dev < 64) attr_set[dev] = true;
             }
             const long n_items = (long)grid;
             const unsigned pgrid = (unsigned)(n_items < 512 ? n_items : 512); // two blocks per CU stay resident
-            hipLaunchKernelGGL((fixed_mfma_db_kernel<3, 3, 2>), dim3(pgrid), dim3(256), lds2, stream, xq16, wq16, wp16, out,
-                               q, (int)n_items);
+            if (pb == 1)
+                hipLaunchKernelGGL((fixed_mfma_db_kernel<3, 3, 1>), dim3(pgrid), dim3(256), lds2, stream, xq16, wq16, wp16,
+                                   out, q, (int)n_items);
+            else
+                hipLaunchKernelGGL((fixed_mfma_db_kernel<3, 3, 2>), dim3(pgrid), dim3(256), lds2, stream, xq16, wq16, wp16,
+                                   out, q, (int)n_items);
             REXSC_CHECK_HIP(hipGetLastError());
             return REXSC_OK;
         }
