@@ -73,12 +73,15 @@ def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_con
                       int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w))
     L = _lib.lib()
     with torch.cuda.device(x.device):
-        ws_bytes = L.rexsc_conv2d_workspace_bytes(ctypes.byref(d))
-        if ws_bytes == 0:
-            _lib.check(-1, "rexsc_conv2d (planning)")
         Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
         Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
         shape = (N, O, Ho, Wo)
+        if N == 0 and Ho > 0 and Wo > 0:  # an empty batch has an empty result; nothing to launch
+            mk = lambda want: _empty_out(shape, torch.int16, x.device, cl_a) if want else None
+            return mk(want_split), mk(want_split), mk(want_diff)
+        ws_bytes = L.rexsc_conv2d_workspace_bytes(ctypes.byref(d))
+        if ws_bytes == 0:
+            _lib.check(-1, "rexsc_conv2d (planning)")
         pos = _empty_out(shape, torch.int16, x.device, cl_a) if want_split else None
         neg = _empty_out(shape, torch.int16, x.device, cl_a) if want_split else None
         diff = _empty_out(shape, torch.int16, x.device, cl_a) if want_diff else None
@@ -101,6 +104,9 @@ def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config):
     d = _lib.LinearDesc(B, C, O, int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
                         int(prog_load[0]), int(prog_load[1]), int(prog_load[2]))
     L = _lib.lib()
+    if B == 0:
+        return (torch.empty((0, O), dtype=torch.int32, device=x.device),
+                torch.empty((0, O), dtype=torch.int32, device=x.device))
     with torch.cuda.device(x.device):
         ws_bytes = L.rexsc_linear_workspace_bytes(ctypes.byref(d))
         if ws_bytes == 0:
@@ -125,11 +131,13 @@ def fixed_conv2d(x, w, add_config, precision_in, precision_out, padding, stride)
                        int(add_config), int(precision_in), int(precision_out))
     L = _lib.lib()
     with torch.cuda.device(x.device):
+        Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
+        Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
+        if N == 0 and Ho > 0 and Wo > 0:
+            return torch.empty((0, O, Ho, Wo), dtype=torch.int32, device=x.device)
         ws_bytes = L.rexsc_fixed_conv2d_workspace_bytes(ctypes.byref(d))
         if ws_bytes == 0:
             _lib.check(-1, "rexsc_fixed_conv2d (planning)")
-        Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
-        Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
         out = torch.empty((N, O, Ho, Wo), dtype=torch.int32, device=x.device)
         ws = _workspace(ws_bytes, x.device)
         rc = L.rexsc_fixed_conv2d(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(out), _ptr(ws), ws.numel(), _stream())

@@ -172,6 +172,31 @@ def test_conv_rejects_bad_arguments():
                                                            True, False)
 
 
+def test_empty_batch_gives_empty_results():
+    """N = 0 (B = 0) is not an error: the ops return empty tensors of the right shape, dtype and device."""
+    import fixed_extension_cuda
+    import sc_extension
+    import sc_extension_cuda
+    import sc_functional as uf
+    w = torch.rand(4, 8, 3, 3, device="cuda")
+    x = torch.rand(0, 8, 6, 6, device="cuda").contiguous(memory_format=torch.channels_last)
+    pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(x, w, 32, -1, 16, (1, 1), (2, 2), (7, 8, 1), 1, 1,
+                                                                  True, False)
+    assert pos.shape == neg.shape == (0, 4, 3, 3) and pos.dtype == torch.int16 and pos.is_cuda
+    assert sc_extension_cuda.conv2d_generic_general_acc(x, w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1, True,
+                                                        False).shape == (0, 4, 6, 6)
+    lp, ln = sc_extension.linear_generic_general(torch.rand(0, 40, device="cuda"), torch.rand(5, 40, device="cuda"),
+                                                 (7, 8, 1), 32, -1, 1, 1, True, False)
+    assert lp.shape == ln.shape == (0, 5) and lp.dtype == torch.int32
+    y = fixed_extension_cuda.conv2d_saturate_acc(x, w, 0, 5, 24, (1, 1), (1, 1))
+    assert y.shape == (0, 4, 6, 6) and y.dtype == torch.int32
+    for sync in (1, 3):
+        out = uf.conv2d_generic(x.requires_grad_(False), w.clone().requires_grad_(True), (1, 1), (1, 1), bit_length=32,
+                                generator="lfsr", forward="or_2", sync=sync, order=5)
+        assert out.shape == (0, 4, 6, 6)
+    assert uf.quantize(x, 7).shape == x.shape
+
+
 RANDOM_FIXED = [
     # N, C, H, W, O, KH, KW, stride, padding, add_config, pin, pout
     (2, 64, 14, 14, 64, 3, 3, (1, 1), (1, 1), 0, 5, 24),     # int8 MFMA closed form, ResNet-like
