@@ -196,6 +196,20 @@ def pointwise(torch, dev):
             ("orn_bias_std_both_backward", lambda: _ops.orn_bias_std_both_backward(gout, x, x2, coef, 2), 20)):
         sec = _time(torch, fn, 20, 3)
         res[name] = {"ms": sec * 1e3, "GB_per_s": bpe * n / sec / 1e9, "hbm_frac": bpe * n / sec / HBM_PEAK}
+    # the kernels of the merged surrogate: both polarities in one [pixels][2][channels] tensor
+    outer, inner = 64 * 56 * 56, 64
+    s2 = (torch.rand(64, 2 * inner, 56, 56, device=dev) * 4).contiguous(memory_format=torch.channels_last)
+    g4 = gout.view(64, 56, 56, inner).permute(0, 3, 1, 2)
+    pos = torch.randint(0, 64, (64, inner, 56, 56), device=dev, dtype=torch.int16).contiguous(memory_format=torch.channels_last)
+    neg = torch.randint(0, 64, (64, inner, 56, 56), device=dev, dtype=torch.int16).contiguous(memory_format=torch.channels_last)
+    for name, fn, bpe in (
+            ("orn_pair_backward", lambda: _ops.orn_pair_backward(g4, s2, outer, inner, True, 2), 20),
+            ("orn_bias_std_pair_forward", lambda: _ops.orn_bias_std_pair_forward(s2, outer, inner, True, coef, coef, 2), 12),
+            ("orn_bias_std_pair_backward", lambda: _ops.orn_bias_std_pair_backward(g4, s2, outer, inner, True, coef, 2), 20),
+            ("sc_counts_to_float", lambda: _ops.sc_counts_to_float(pos, neg, 32), 8),
+            ("quantize", lambda: _ops.quantize(x, 7), 8)):
+        sec = _time(torch, fn, 20, 3)
+        res[name] = {"ms": sec * 1e3, "GB_per_s": bpe * n / sec / 1e9, "hbm_frac": bpe * n / sec / HBM_PEAK}
     return res
 
 
