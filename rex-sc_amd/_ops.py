@@ -377,6 +377,23 @@ def sc_counts_to_float(pos, neg, bit_length):
     return y
 
 
+def storage_flat(t, channels_last):
+    """1-D view of a dense 4-D tensor in the order of its storage (2-D tensors: row major)."""
+    if t.dim() == 4 and channels_last:
+        return t.permute(0, 2, 3, 1).reshape(-1)
+    return t.reshape(-1)
+
+
+def sc_counts_pair(pos, neg, bit_length, outer, inner, channels_last):
+    """float(pos) / L and float(neg) / L of one SC conv call laid out like the merged surrogate's sums,
+    [outer][2][inner] (calibration only: plain torch ops)."""
+    if channels_last:
+        p2, n2 = pos.permute(0, 2, 3, 1).reshape(outer, inner), neg.permute(0, 2, 3, 1).reshape(outer, inner)
+    else:
+        p2, n2 = pos.reshape(outer, inner), neg.reshape(outer, inner)
+    return torch.stack((p2, n2), dim=1).to(torch.float32).div_(bit_length)
+
+
 def _weight_geometry(w):
     """(dense float32 w, O, C, taps, channels_last) of a conv [O,C,KH,KW] or linear [O,C] weight."""
     wd = _dense_f32(w)

@@ -213,6 +213,16 @@ def compute_bias_std_coef(or_n, a_bit, a_act, order):
 
 
 # ---- merged surrogate ---------------------------------------------------------------------------
+def merged_surrogate_sums(activation, weight, pad_hw, stride):
+    """One convolution with the 2*O filters [w_pos ; w_neg], written in the activation's memory order (no
+    conversion pass inside the convolution): -> (w2, s2, outer, inner, channels_last) with s2 laid out
+    [outer][2][inner]."""
+    with torch.no_grad():
+        w2 = _ops.split_weight(weight, channels_last=_ops.is_channels_last(activation))
+        s2, outer, inner, cl = _ops.pair_layout(F.conv2d(activation.detach(), w2, padding=pad_hw, stride=stride))
+    return w2, s2, outer, inner, cl
+
+
 class Merged_Surrogate_Conv(torch.autograd.Function):
     """The float surrogate of conv2d_generic for forward = 'or_n' (n <= 4) / 'full_or' with its two
     convolutions merged: one conv with the 2*O filters [clamp(w, 0, 100) ; -clamp(w, -100, 0)]
@@ -221,18 +231,21 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
 
     sync = 1: the forward value is the SC result `sc_value` (= pos / L - neg / L, the tensor the
     reference writes into `.data`, :1273-1274) and the OR-n forward is never evaluated;
-    sync = 3: the forward value is the fused OR-n + bias/noise kernel's (:1253-1254).
-    Gradients are those of OR_n(conv(x, w_pos)) - OR_n(conv(x, w_neg)) (sync 3: with the bias
+    sync = 3: the forward value is the fused OR-n + bias/noise kernel's (:1253-1254);
+    sync = 2: the caller has fitted the bias / std polynomials to SC result - OR_n(sum) on the sums it
+    passes in (`sums`, :1275-1283); the forward value is Bias_Correct(OR_n(sum_pos)) -
+    Bias_Correct(OR_n(sum_neg)) with those coefficients (:1284-1285), which is what the sync-3 kernel computes.
+    Gradients are those of OR_n(conv(x, w_pos)) - OR_n(conv(x, w_neg)) (sync 2, 3: with the bias
     polynomial's derivative), evaluated on the saved sums rounded to binary16 as the reference's
     backward wrappers do."""
 
     @staticmethod
-    def forward(ctx, activation, weight, sc_value, bias_coef, std_coef, or_n, pad_hw, stride, sync):
-        # the filters are written in the activation's memory order: no conversion pass inside the convolutions
-        w2 = _ops.split_weight(weight, channels_last=_ops.is_channels_last(activation))
-        s2, outer, inner, cl = _ops.pair_layout(F.conv2d(activation, w2, padding=pad_hw, stride=stride))
+    def forward(ctx, activation, weight, sc_value, bias_coef, std_coef, or_n, pad_hw, stride, sync, sums):
+        if sums is None:
+            sums = merged_surrogate_sums(activation, weight, pad_hw, stride)
+        w2, s2, outer, inner, cl = sums
         ctx.geom = (outer, inner, cl, or_n, tuple(pad_hw), tuple(stride), sync)
-        if sync == 3:
+        if sync >= 2:
             ctx.save_for_backward(activation, weight, w2, s2, bias_coef)
             return _ops.orn_bias_std_pair_forward(s2, outer, inner, cl, bias_coef, std_coef, or_n)
         ctx.save_for_backward(activation, weight, w2, s2)
@@ -241,7 +254,7 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         outer, inner, cl, or_n, pad_hw, stride, sync = ctx.geom
-        if sync == 3:
+        if sync >= 2:
             activation, weight, w2, s2, bias_coef = ctx.saved_tensors
             g2 = _ops.orn_bias_std_pair_backward(grad_output, s2, outer, inner, cl, bias_coef, or_n)
         else:
@@ -254,7 +267,7 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
                                                              (0, 0), 1, (need_x, need_w, False))
             if need_w:
                 dw = _ops.merge_weight_grad(dw2, weight).to(weight.dtype)
-        return dx, dw, None, None, None, None, None, None, None
+        return dx, dw, None, None, None, None, None, None, None, None
 
 
 class Merged_Surrogate_Linear(torch.autograd.Function):
@@ -306,6 +319,9 @@ def _merged_surrogate_ok(activation, weight, forward, or_n, sync, sc_on, split_o
             return False
     elif sync == 3:
         if not (forward[:3] == "or_" and len(forward) == 4):
+            return False
+    elif sync == 2:
+        if not sc_on or not (forward[:3] == "or_" and len(forward) == 4):
             return False
     else:
         return False
@@ -379,9 +395,24 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     if (sync_override == 3 or has_sc_kernel) and _merged_surrogate_ok(
             activation, weight, forward, or_n, sync_override, sc_on, split_output, stride, pad_hw):
         n = 1 if forward in ("full_or", "and_2") else or_n
-        if sync_override != 1:
-            return Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride,
-                                               sync_override)
+        if sync_override == 3:
+            return Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride, 3, None)
+        if sync_override == 2:
+            with torch.no_grad():
+                pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(
+                    activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
+                    (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
+                sums = merged_surrogate_sums(activation, weight, pad_hw, stride)
+                _, s2, outer, inner, cl = sums
+                # calibration: a_act = OR_n of both sums (one pass over the pair tensor), a_bit = the SC
+                # results in the same element order
+                a_act = _ops.storage_flat(_ops.orn_forward(s2, n), cl)
+                a_bit = _ops.sc_counts_pair(pos, neg, bit_length, outer, inner, cl).reshape(-1)
+                bias_new, std_new = compute_bias_std_coef(or_n, a_bit, a_act, order)
+                bias_coef[:bias_new.size(0)] = bias_new
+                std_coef[:std_new.size(0)] = std_new
+            out = Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride, 2, sums)
+            return out, bias_coef, std_coef
 
         def sc_forward():
             with torch.no_grad():
@@ -397,12 +428,12 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
         side = _side_stream(activation.device)
         if side is None:
             return Merged_Surrogate_Conv.apply(activation, weight, sc_forward(), bias_coef, std_coef, n, pad_hw,
-                                               stride, 1)
+                                               stride, 1, None)
         cur = torch.cuda.current_stream(activation.device)
         side.wait_stream(cur)
         with torch.cuda.stream(side):
             sc_value = sc_forward()
-        out = Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride, 1)
+        out = Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride, 1, None)
         cur.wait_stream(side)
         sc_value.record_stream(cur)  # allocated on the side stream, consumed on the caller's
         return out

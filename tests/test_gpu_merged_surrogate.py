@@ -186,3 +186,36 @@ def test_linear_merged_equals_two_gemms(forward, monkeypatch):
     assert torch.equal(res[0][0], res[1][0])
     _close(res[0][1], res[1][1], "grad x")
     _close(res[0][2], res[1][2], "grad w")
+
+
+@pytest.mark.parametrize("cl", [False, True])
+def test_sync2_merged_equals_two_convolutions(cl, monkeypatch):
+    """Calibration step: same fitted polynomials, same gradients; the forward values differ only by the
+    noise realisation (another generator), so their difference is zero-mean with the fitted spread."""
+    import sc_functional as uf
+    x, w = _operands(27, 4, 32, 16, 16, 32, 3, dens=0.3)
+    res = []
+    for merged in ("1", "0"):
+        monkeypatch.setenv("REXSC_MERGED_SURROGATE", merged)
+        xt = x.cuda()
+        if cl:
+            xt = xt.contiguous(memory_format=torch.channels_last)
+        xt.requires_grad_(True)
+        wt = w.cuda().requires_grad_(True)
+        bias, std = torch.zeros(6, device="cuda"), torch.zeros(6, device="cuda")
+        torch.manual_seed(3)
+        out, b2, s2 = uf.conv2d_generic(xt, wt, (1, 1), (1, 1), bit_length=32, generator="lfsr", forward="or_2", sync=2,
+                                        order=5, bias_coef=bias, std_coef=std)
+        assert b2 is bias and s2 is std and std.abs().sum() > 0   # updated in place (the bias fit may be suppressed)
+        g = torch.randn(out.shape, generator=torch.Generator().manual_seed(5)).cuda()
+        out.backward(g)
+        res.append((out.detach().cpu().double(), xt.grad.cpu(), wt.grad.cpu(), bias.cpu(), std.cpu()))
+    (ya, gxa, gwa, ba, sa), (yb, gxb, gwb, bb, sb) = res
+    xs = torch.linspace(0, 1.5, 16)
+    poly = lambda c: sum(float(c[i]) * xs ** i for i in range(6))
+    assert torch.allclose(poly(ba), poly(bb), atol=2e-4) and torch.allclose(poly(sa), poly(sb), atol=2e-4)
+    _close(gxa, gxb, "grad x")
+    _close(gwa, gwb, "grad w")
+    d = ya - yb
+    spread = float(d.std())
+    assert 0 < spread < 0.5 and abs(float(d.mean())) < 6 * spread / d.numel() ** 0.5
