@@ -6,7 +6,7 @@
  * All return 0 on success and a negative code on failure; rexsc_last_error() returns the
  * message of the calling thread's last failure.  Nothing here allocates device memory:
  * ops that need scratch take a caller-owned workspace whose size the matching
- * *_workspace_bytes() call reports.  Inputs are never written.  Work is enqueued on
+ * *_workspace_bytes() call reports (rexsc_conv2d_orn_noalloc uses a static device array instead).  Inputs are never written.  Work is enqueued on
  * `stream` and the call returns without synchronising.
  *
  * Each entry point names the reference interface it replaces (paths relative to the
@@ -75,6 +75,18 @@ int rexsc_conv2d_plan_info(const rexsc_conv_desc *d, int64_t *out);
 int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const float *w,
                      int16_t *out_pos, int16_t *out_neg, int16_t *out_diff,
                      void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
+/* The same op for callers that cannot allocate device memory or hand over a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  The workspace is a static device array inside the library
+ * (REXSC_NOALLOC_SCRATCH_BYTES, held on every GPU the library runs on until the process ends); the
+ * call makes no hipMalloc / hipFree and calls no allocating routine.  Problems whose workspace
+ * (rexsc_conv2d_workspace_bytes) exceeds the array are rejected with REXSC_ERR_WORKSPACE.  All calls
+ * on one GPU share the array: calls that overlap on one GPU (different streams or threads) race.
+ * Call rexsc_init() once per device before the first call that runs under stream capture. */
+#define REXSC_NOALLOC_SCRATCH_BYTES (32u << 20)
+int rexsc_conv2d_orn_noalloc(const rexsc_conv_desc *d, const float *x, const float *w,
+                             int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, rexsc_stream_t stream);
 
 /* ---- SC linear -------------------------------------------------------------------------
  * Replaces sc_extension_cuda.linear_generic_general_acc (sc_cuda.cpp:101-120) and

@@ -8,6 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "librexsc.so")
+NOALLOC_SCRATCH_BYTES = 32 << 20  # REXSC_NOALLOC_SCRATCH_BYTES of include/rexsc.h
 _lib = None
 
 
@@ -48,6 +49,7 @@ SIGNATURES = {
     "rexsc_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(ConvDesc)]),
     "rexsc_conv2d_plan_info": (_int, [ctypes.POINTER(ConvDesc), ctypes.POINTER(ctypes.c_int64)]),
     "rexsc_conv2d_orn": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_conv2d_orn_noalloc": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp]),
     "rexsc_linear_workspace_bytes": (_sz, [ctypes.POINTER(LinearDesc)]),
     "rexsc_linear_orn": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "rexsc_orn_forward": (_int, [_vp, _vp, _sz, _int, _vp]),

@@ -10,6 +10,7 @@
 //  * sequential (add_config >= 1): the OR-style adders are order dependent and are evaluated
 //    product by product in the reference's (c, ky, kx) order.
 #include <stdlib.h>
+#include <atomic>
 #include "profile.h"
 #include "rexsc_common.h"
 
@@ -693,7 +694,7 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         const size_t lds = (size_t)2 * q.KH * q.KW * 2 * FT * 16;
         ProfScope prof("fixed_conv_mfma", io_bytes, stream);
         if (db_shape) {
-            static bool attr_set[64] = {}; // per device: the kernel needs more than the default 64 KB of LDS
+            static std::atomic<bool> attr_set[64]; // zero-initialised; per device: the kernel needs more than the default 64 KB of LDS
             const size_t lds2 = 2 * lds;
             int dev = 0;
             REXSC_CHECK_HIP(hipGetDevice(&dev));

@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <stdlib.h>
 #include <string.h>
+#include <mutex>
 
 #include "sc_compute.h"
 #include "sng.h"
@@ -242,6 +243,76 @@ int plan_linear(ScPlan &pl, const rexsc_linear_desc *d)
     return REXSC_OK;
 }
 
+// ---- scratch of the entry point that allocates nothing ------------------------------------------
+// rexsc_conv2d_orn_noalloc() carves its workspace (weight streams, activation streams, split
+// partials, state-plane table) out of this array instead of a caller-owned buffer.  Every GPU the
+// library runs on holds its own copy until the process ends.  In host code the array's name is only a
+// handle for hipGetSymbolAddress: the address kernels may use is resolved once per device
+// (static_scratch) and that pointer is what is carved up and passed to the kernels.
+static __device__ __align__(256) unsigned char scratch[REXSC_NOALLOC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+
+int static_scratch(void **out)
+{
+    static std::mutex mu;
+    static void *dev_ptr[MAX_DEVICES] = {nullptr};
+    int dev = 0;
+    REXSC_CHECK_HIP(hipGetDevice(&dev));
+    REXSC_CHECK_ARG(dev >= 0 && dev < MAX_DEVICES, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!dev_ptr[dev]) {
+        void *p = nullptr;
+        REXSC_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        REXSC_CHECK_ARG(p != nullptr && ((uintptr_t)p % WS_ALIGN) == 0, "static scratch has no usable device address");
+        dev_ptr[dev] = p;
+    }
+    *out = dev_ptr[dev];
+    return REXSC_OK;
+}
+
+// The conv op proper: generators, compute, finalize, batch chunk by batch chunk, in `workspace`
+// (device memory of at least pl.total bytes).
+int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
+             int16_t *out_neg, int16_t *out_diff, void *workspace, hipStream_t stream)
+{
+    uint8_t *ws = (uint8_t *)workspace;
+    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
+    uint32_t *A = (uint32_t *)(ws + pl.off_a);
+    uint32_t *part = (uint32_t *)(ws + pl.off_part);
+    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
+
+    int rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+    if (rc) return rc;
+    const size_t in_image = (size_t)d->C * d->H * d->W;
+    const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
+    for (int n0 = 0; n0 < d->N; n0 += pl.n_chunk) {
+        const int nc = d->N - n0 < pl.n_chunk ? d->N - n0 : pl.n_chunk;
+        ActGeom ag = pl.ag;
+        ComputeParams cp = pl.cp;
+        ag.N = nc;
+        cp.M = nc * pl.Ho * pl.Wo; // slot stride keeps the full-chunk value: the buffer is laid out for n_chunk images
+        rc = sng_activations(x + n0 * in_image, A, tab_a, ag, pl.gen_act, stream);
+        if (rc) return rc;
+        int16_t *op = out_pos ? out_pos + n0 * out_image : nullptr;
+        int16_t *on = out_neg ? out_neg + n0 * out_image : nullptr;
+        int16_t *od = out_diff ? out_diff + n0 * out_image : nullptr;
+        if (!pl.tuned) {
+            rc = sc_compute_generic(A, Wst, cp, pl.KW, pl.ZC, op, on, od, stream);
+            if (rc) return rc;
+            continue;
+        }
+        rc = sc_compute(A, Wst, cp, pl.KW, pl.ZC, false, part, op, on, od, stream);
+        if (rc) return rc;
+        if (!cp.direct) {
+            cp.m_tiles = cp.o_tiles = 0;
+            rc = sc_finalize_i16(part, cp, op, on, od, stream);
+            if (rc) return rc;
+        }
+    }
+    return REXSC_OK;
+}
+
 } // namespace
 } // namespace rexsc
 
@@ -253,7 +324,10 @@ extern "C" int rexsc_version(void) { return 100; }
 extern "C" int rexsc_init(rexsc_stream_t stream)
 {
     const SeqTable *t = nullptr;
-    return get_seq_tables(&t, (hipStream_t)stream);
+    int rc = get_seq_tables(&t, (hipStream_t)stream);
+    if (rc) return rc;
+    void *ws = nullptr;
+    return static_scratch(&ws); // device address of the no-alloc entry point's scratch array
 }
 
 extern "C" size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d)
@@ -291,41 +365,32 @@ extern "C" int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const 
         set_error("conv2d: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
         return REXSC_ERR_WORKSPACE;
     }
-    uint8_t *ws = (uint8_t *)workspace;
-    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
-    uint32_t *A = (uint32_t *)(ws + pl.off_a);
-    uint32_t *part = (uint32_t *)(ws + pl.off_part);
-    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
+    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, workspace, stream);
+}
 
-    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+// Same op with the workspace taken from the library's static device array: no allocation of any kind,
+// for callers that cannot allocate (HIP graph capture, tight serving loops).  Calls that overlap on
+// one GPU share that array and race.
+extern "C" int rexsc_conv2d_orn_noalloc(const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
+                                        int16_t *out_neg, int16_t *out_diff, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_conv(pl, d);
     if (rc) return rc;
-    const size_t in_image = (size_t)d->C * d->H * d->W;
-    const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
-    for (int n0 = 0; n0 < d->N; n0 += pl.n_chunk) {
-        const int nc = d->N - n0 < pl.n_chunk ? d->N - n0 : pl.n_chunk;
-        ActGeom ag = pl.ag;
-        ComputeParams cp = pl.cp;
-        ag.N = nc;
-        cp.M = nc * pl.Ho * pl.Wo; // slot stride keeps the full-chunk value: the buffer is laid out for n_chunk images
-        rc = sng_activations(x + n0 * in_image, A, tab_a, ag, pl.gen_act, stream);
-        if (rc) return rc;
-        int16_t *op = out_pos ? out_pos + n0 * out_image : nullptr;
-        int16_t *on = out_neg ? out_neg + n0 * out_image : nullptr;
-        int16_t *od = out_diff ? out_diff + n0 * out_image : nullptr;
-        if (!pl.tuned) {
-            rc = sc_compute_generic(A, Wst, cp, pl.KW, pl.ZC, op, on, od, stream);
-            if (rc) return rc;
-            continue;
-        }
-        rc = sc_compute(A, Wst, cp, pl.KW, pl.ZC, false, part, op, on, od, stream);
-        if (rc) return rc;
-        if (!cp.direct) {
-            cp.m_tiles = cp.o_tiles = 0;
-            rc = sc_finalize_i16(part, cp, op, on, od, stream);
-            if (rc) return rc;
-        }
+    REXSC_CHECK_ARG(x && w, "null operand pointer");
+    REXSC_CHECK_ARG(out_pos || out_neg || out_diff, "no output pointer given");
+    if (pl.total > (size_t)REXSC_NOALLOC_SCRATCH_BYTES) {
+        set_error("conv2d (no-alloc): this problem needs %zu bytes of scratch, the static array holds %zu; use "
+                  "rexsc_conv2d_orn with a caller-owned workspace", pl.total, (size_t)REXSC_NOALLOC_SCRATCH_BYTES);
+        return REXSC_ERR_WORKSPACE;
     }
-    return REXSC_OK;
+    void *ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc) return rc;
+    // Nothing in the workspace has to start at zero: the generators write every word the compute
+    // kernel uses, and the finalize pass reads only partials the compute kernel has just written.
+    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, ws, stream);
 }
 
 extern "C" size_t rexsc_linear_workspace_bytes(const rexsc_linear_desc *d)

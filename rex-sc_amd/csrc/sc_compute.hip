@@ -18,6 +18,8 @@
 //                     and 3 resident waves each, whole-reduction waves would quantise badly.
 //   grid            = pixel tiles x output-channel tiles x (optional) global slot splits, remapped
 //                     so that the blocks sharing a pixel tile run on the same XCD (shared L2).
+#include <string>
+
 #include "sc_compute.h"
 #include "profile.h"
 
@@ -527,8 +529,13 @@ static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams 
     const long blocks = (long)p.m_tiles * p.o_tiles * p.splits;
     REXSC_CHECK_ARG(blocks < (1L << 30), "SC compute: grid too large (%ld blocks)", blocks);
     const int grid = (int)align_up((size_t)blocks, 8);
-    static char name[64] = "";
-    if (!name[0]) snprintf(name, sizeof(name), "sc_compute<%d,%d,%d,%d,%d>", KW, ZC, PX, OT, MODE);
+    // built once per instance; initialisation of a function-local static is thread-safe
+    static const std::string name_str = [] {
+        char b[64];
+        snprintf(b, sizeof(b), "sc_compute<%d,%d,%d,%d,%d>", KW, ZC, PX, OT, MODE);
+        return std::string(b);
+    }();
+    const char *name = name_str.c_str();
     // algorithmic lane-ops: (and + popcount-accumulate) x 2 polarities per 32-channel word
     ProfScope prof(name, 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
     hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, MODE>), dim3(grid), dim3(64 * p.ns), 0, stream, A, Wst, p, part,

@@ -12,6 +12,7 @@
 // (linear); quantisation sc_conv.cpp:316-320.
 #include <stdlib.h>
 #include <string.h>
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -41,11 +42,18 @@ __global__ void build_seq_tables_kernel()
 
 int get_seq_tables(const SeqTable **tables, hipStream_t stream)
 {
+    static std::mutex mu;
     static SeqTable *dev_ptr[64] = {nullptr};
     int dev = 0;
     REXSC_CHECK_HIP(hipGetDevice(&dev));
     REXSC_CHECK_ARG(dev >= 0 && dev < 64, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
     if (!dev_ptr[dev]) {
+        // The one-time build ends with a synchronisation, which a stream under capture cannot take.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        REXSC_CHECK_HIP(hipStreamIsCapturing(stream, &cap));
+        REXSC_CHECK_ARG(cap == hipStreamCaptureStatusNone,
+                        "first use on this device while the stream is being captured: call rexsc_init() before the capture");
         SeqTable *p = nullptr;
         REXSC_CHECK_HIP(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(g_seq_tables)));
         hipLaunchKernelGGL(build_seq_tables_kernel, dim3(1), dim3(64), 0, stream);
