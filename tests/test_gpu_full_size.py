@@ -41,8 +41,24 @@ def test_config2_linear_or2_full_size_exact():
     assert np.array_equal(pos.cpu().numpy(), opos) and np.array_equal(neg.cpu().numpy(), oneg)
 
 
+# all ten distinct SC layer shapes of ResNet-18 at 224x224 (C_in, H_in, C_out, K, stride)
+def test_config2_linear_or2_full_size_dense_operands():
+    """The benchmark's own operand distribution (dense weights): every OR-2 count saturates, so almost every
+    output is 2 * 64 -- the all-saturated path, exact against the oracle."""
+    import sc_extension
+    g = torch.Generator().manual_seed(2)
+    x = torch.randint(0, 64, (256, 4096), generator=g).float() / 64
+    w = ((torch.rand(1024, 4096, generator=g) * 2 - 1) * 64).round().clamp(-63, 63) / 64
+    print("config2 full, dense", flush=True)
+    pos, neg = sc_extension.linear_generic_general(x.cuda(), w.cuda(), (7, 8, 1), 64, -1, 1, 1, True, False)
+    opos, oneg = orc.linear_generic_general(x.numpy(), w.numpy(), (7, 8, 1), 64, -1, 1, 1)
+    assert opos.max() == 128 and (opos == 128).mean() > 0.5
+    assert np.array_equal(pos.cpu().numpy(), opos) and np.array_equal(neg.cpu().numpy(), oneg)
+
+
 STAGES = [(64, 56, 64, 3, 1), (64, 56, 128, 3, 2), (64, 56, 128, 1, 2), (128, 28, 128, 3, 1),
-          (256, 14, 256, 3, 1), (512, 7, 512, 3, 1)]
+          (128, 28, 256, 3, 2), (128, 28, 256, 1, 2), (256, 14, 256, 3, 1),
+          (256, 14, 512, 3, 2), (256, 14, 512, 1, 2), (512, 7, 512, 3, 1)]
 
 
 @pytest.mark.parametrize("shape", STAGES, ids=lambda s: "c%d_h%d_o%d_k%d_s%d" % s)

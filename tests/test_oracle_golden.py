@@ -12,12 +12,13 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 class _Golden:
-    """The two fixtures written by the reference's compiled CPU extension: hand-picked cases
-    (make_golden.py) and seeded random configurations (make_golden_random.py), as one key space."""
+    """The fixtures written by the reference's compiled CPU extension: hand-picked cases (make_golden.py),
+    seeded random configurations (make_golden_random.py) and operands off the quantisation grid
+    (make_golden_offgrid.py), as one key space."""
 
     def __init__(self):
         self.files = [np.load(os.path.join(ROOT, "tests", "golden", f), allow_pickle=False)
-                      for f in ("ref_cpu_ext.npz", "ref_cpu_ext_random.npz")]
+                      for f in ("ref_cpu_ext.npz", "ref_cpu_ext_random.npz", "ref_cpu_ext_offgrid.npz")]
         self.meta = {"conv": [], "linear": [], "fixed": []}
         for f in self.files:
             m = json.loads(bytes(f["meta"]).decode())
