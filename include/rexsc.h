@@ -45,6 +45,7 @@ int rexsc_init(rexsc_stream_t stream);
  * 2^lfsr_length when lfsr_length > 0), clamped and ceil'ed to integers, expanded to LFSR
  * bitstreams (XOR-feedback LFSR, seeds 1..2^lb-1), AND-multiplied, popcounted over the whole
  * Cin*KH*KW reduction per stream cycle, clamped to n_sat per cycle and summed over cycles.
+ * desc.xnor = 1 switches the stream generators to those of the reference's CUDA kernels.
  */
 typedef struct rexsc_conv_desc {
     int32_t N, C, H, W;          /* activation dims, UNPADDED */
@@ -58,6 +59,10 @@ typedef struct rexsc_conv_desc {
     int32_t total_width, load_width, load_wait; /* progressive loading (7,8,1 = off) */
     int32_t act_channels_last;   /* memory order of x: 0 NCHW, 1 NHWC; outputs use the same order */
     int32_t weight_channels_last;/* memory order of w: 0 OIHW, 1 OHWI */
+    int32_t xnor;                /* 0: the CPU extension's generator (it ignores its xnor argument, sc_conv.cpp:362-425);
+                                  * 1: the generator of the reference's CUDA conv kernels called with xnor = true
+                                  *    (sc_cuda_conv.cu:28,55-56,139; sc_device.cuh:108-286): XNOR-feedback LFSR,
+                                  *    seeds (index % (2^lb-1)) + 0, the same LFSR for gen_config 2; lb <= 7 */
 } rexsc_conv_desc;
 
 size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d);

@@ -89,13 +89,16 @@ def _pad_hw(x, padding):
 
 def conv2d_generic_general_split(x, w, bit_length, lfsr_length, z_units, padding, stride, prog_load,
                                  bin_config, gen_config, xnor=False, mux=False,
-                                 channels_last_activation=False, channels_last_weight=False):
+                                 channels_last_activation=False, channels_last_weight=False, cuda_xnor=False):
     """sc_conv.cpp:301-489, returning (pos, neg) int16 in logical NCHW index order.
 
     x [N,C,H,W] and w [O,C,KH,KW] are float arrays in logical NCHW/OIHW index order; the two
     flags say which memory order the reference would have seen (they only select the
     operand/ output index formulas, the returned arrays are always logical NCHW).
-    xnor and mux are accepted and ignored, as in the reference CPU extension.
+    xnor and mux are accepted and ignored, as in the reference CPU extension; cuda_xnor=True instead
+    restates the stream generators of the reference's CUDA kernels called with xnor=True
+    (sc_cuda_conv.cu:28,55-56,139): XNOR-feedback LFSR, seeds lowered by one (no CUDA build or
+    fixture exists; pinned by invariants and a per-bit brute force, tests/test_oracle_invariants.py).
     """
     x = np.asarray(x, dtype=np.float32)
     w = np.asarray(w, dtype=np.float32)
@@ -118,7 +121,7 @@ def conv2d_generic_general_split(x, w, bit_length, lfsr_length, z_units, padding
     rc = lib().orc_conv2d(_p(xq, _i32p), _p(wp, _i32p), _p(wn, _i32p), _p(pos, _i16p), _p(neg, _i16p),
                           N, C, H, W, O, KH, KW, s0, s1, int(bit_length), int(lfsr_length), int(gen_config),
                           int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(bin_config),
-                          int(channels_last_activation), int(channels_last_weight))
+                          int(channels_last_activation), int(channels_last_weight), int(bool(cuda_xnor)))
     if rc != 0:
         raise ValueError("oracle conv2d: unsupported configuration (rc=%d)" % rc)
     if channels_last_activation:

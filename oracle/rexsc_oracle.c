@@ -16,6 +16,9 @@
  *   orc_quantize_*           closed form on grids + golden outputs (indirect)
  *   orc_conv2d               golden outputs of the compiled reference + dense {0,1} conv
  *                            special case + OR-1 "any" special case
+ *   orc_conv2d, xnor = 1     (generators of the reference's CUDA kernels; no CUDA build or fixture
+ *                            exists) LFSR cycle / complement invariants + per-bit brute-force model
+ *                            written from sc_cuda_conv.cu, tests/test_oracle_invariants.py
  *   orc_linear               golden outputs of the compiled reference + matmul special case
  *   orc_fixed_conv2d         golden outputs of the compiled reference + closed form
  *   orc_orn_* / orc_bias_*   analytic closed forms in float64 (forward and derivative)
@@ -32,11 +35,13 @@
  * LFSR steps.  sc_cpu.hpp:49-190.  Fibonacci form: feedback = XOR of the tap bits,
  * next = feedback + 2*(state mod 2^(lb-1)).  Taps (bit positions, MSB = lb-1):
  *   3:{2,1} 4:{3,2} 5:{4,2} 6:{5,4} 7:{6,5} 8:{7,5,4,3}
- * The "_acc" flavour (acc != 0) splices the all-zero state into the cycle: 1 -> 0 -> 2.
+ * Flavours (`acc`): 0 plain; 1 the "_acc" variant, which splices the all-zero state into
+ * the cycle: 1 -> 0 -> 2; 2 the XNOR variant of the reference's CUDA kernels
+ * (sc_device.cuh:108-286, d_lfsr_N_xnor): feedback = 1 - XOR of the tap bits.
  * ---------------------------------------------------------------------------------- */
 int orc_lfsr_step(int lb, int acc, int v)
 {
-    if (acc) {
+    if (acc == 1) {
         if (v == 1) return 0;
         if (v == 0) return 2;
     }
@@ -50,6 +55,7 @@ int orc_lfsr_step(int lb, int acc, int v)
     case 8: fb = ((v >> 7) ^ (v >> 5) ^ (v >> 4) ^ (v >> 3)) & 1; break; /* :49-52 */
     default: return -1;
     }
+    if (acc == 2) fb = 1 - fb;                                /* sc_device.cuh:108,147,172,197,224,244 */
     return fb + 2 * (v & ((1 << (lb - 1)) - 1));
 }
 
@@ -152,6 +158,13 @@ static void orc_sng_group(const int *val, const int *seed, int lb, int acc, int 
  * Per output and polarity: sum over slots of min(popcount total of the slot, n_sat); the
  *        running sum lives in 16 bits and wraps (:25-33, :286-294).
  * n_sat = bin_config+1 if bin_config>=0 else 1-bin_config (:216-224).
+ * xnor = 0: the CPU extension, which ignores its xnor argument.  xnor = 1: the stream generators
+ *        of the reference's CUDA kernels called with xnor = true (sc_cuda_conv.cu:3-166): the
+ *        XNOR LFSR for every gen_config (:28,139 -- the CUDA kernels have no "_acc" variant) and
+ *        seeds lowered by one, (...) % P + 1 - 1 (:55-56,139).  No CUDA build or fixture of the
+ *        reference exists to compare with; pinned by LFSR invariants and a per-bit brute-force
+ *        model written from the CUDA source, tests/test_oracle_invariants.py.  8-bit LFSRs are refused: the CUDA
+ *        kernels keep states and operands in int8 (:37-40).
  * Returns 0, or -1 for an unsupported stream length / generator.
  * ---------------------------------------------------------------------------------- */
 int orc_conv2d(const int32_t *xq, const int32_t *wpos, const int32_t *wneg,
@@ -159,11 +172,13 @@ int orc_conv2d(const int32_t *xq, const int32_t *wpos, const int32_t *wneg,
                int N, int C, int H, int W, int O, int KH, int KW, int s0, int s1,
                int bit_length, int lfsr_length, int gen_config,
                int total_width, int load_width, int load_wait,
-               int bin_config, int cl_act, int cl_w)
+               int bin_config, int cl_act, int cl_w, int xnor)
 {
     const int lb = orc_lfsr_bits(bit_length, lfsr_length);
     if (lb < 0 || gen_config < 1 || gen_config > 2) return -1;
-    const int acc = (gen_config == 2);
+    if (xnor && lb == 8) return -1;
+    const int acc = xnor ? 2 : (gen_config == 2);
+    const int seed_off = xnor ? 0 : 1;
     const int P = (1 << lb) - 1;
     const int Z = (C + ORC_PACK - 1) / ORC_PACK;
     const int g = gen_config;
@@ -191,7 +206,7 @@ int orc_conv2d(const int32_t *xq, const int32_t *wpos, const int32_t *wneg,
                 long wi = cl_w ? (((long)o * KH + ky) * KW + kx) * C + c
                                : (((long)o * C + c) * KH + ky) * KW + kx;
                 vp[cc] = wpos[wi]; vn[cc] = wneg[wi];
-                seed[cc] = (ORC_WEIGHT_SEED + c * KH * KW + ky * KW + kx) % P + 1;
+                seed[cc] = (ORC_WEIGHT_SEED + c * KH * KW + ky * KW + kx) % P + seed_off;
             } else { vp[cc] = vn[cc] = seed[cc] = 0; }
         }
         orc_sng_group(vp, seed, lb, acc, bit_length, total_width, load_width, load_wait, words_p);
@@ -215,7 +230,7 @@ int orc_conv2d(const int32_t *xq, const int32_t *wpos, const int32_t *wneg,
                 long xi = cl_act ? (((long)n * H + y) * W + x) * C + c
                                  : (((long)n * C + c) * H + y) * W + x;
                 v[cc] = xq[xi];
-                seed[cc] = (c * H * W + y * W + x) % P + 1;
+                seed[cc] = (c * H * W + y * W + x) % P + seed_off;
             } else { v[cc] = seed[cc] = 0; }
         }
         orc_sng_group(v, seed, lb, acc, bit_length, total_width, load_width, load_wait, words);

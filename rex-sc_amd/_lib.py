@@ -16,7 +16,7 @@ class ConvDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
         "bit_length", "lfsr_length", "gen_config", "bin_config",
-        "total_width", "load_width", "load_wait", "act_channels_last", "weight_channels_last")]
+        "total_width", "load_width", "load_wait", "act_channels_last", "weight_channels_last", "xnor")]
 
 
 class LinearDesc(ctypes.Structure):

@@ -1,15 +1,45 @@
 """Tensor-level plumbing shared by the drop-in extension modules: layout decisions, workspace,
 stream, and the calls into the C ABI.  PyTorch is used for device memory and streams only."""
 import ctypes
+import os
+import warnings
 
 import torch
 
 import _lib
 
-# How the `xnor` argument of the conv op is treated.  The reference's CPU extension ignores it
-# (XOR-feedback LFSR, seeds 1..2^lb-1; sc_conv.cpp:362-425) while its CUDA kernels switch to an
-# XNOR LFSR.  Bit-exactness is defined against the CPU extension, so that is the only mode built.
-XNOR_MODE = "cpu_oracle"
+# How the `xnor` argument of the conv op is treated (environment variable REXSC_XNOR_MODE, read at call time):
+#   cpu_oracle (default)  ignored, as the reference's CPU extension does (XOR-feedback LFSR, seeds 1..2^lb-1;
+#                         sc_conv.cpp:362-425).  Bit-exactness is defined against that extension.
+#   cuda_ref              honoured, as the reference's CUDA conv kernels do (XNOR-feedback LFSR, seeds lowered by
+#                         one, the same LFSR for the and_2 generator; sc_cuda_conv.cu:28,55-56,139): a caller
+#                         coming from the CUDA extension keeps the bit streams it had.  The linear op has no XNOR
+#                         generator in either reference extension (sc_cuda_matmul.cu:27-57).
+XNOR_MODES = ("cpu_oracle", "cuda_ref")
+_warned_xnor_ignored = False
+
+
+def xnor_mode():
+    mode = os.environ.get("REXSC_XNOR_MODE", "cpu_oracle")
+    if mode not in XNOR_MODES:
+        raise RuntimeError("REXSC_XNOR_MODE must be one of %s (got %r)" % (", ".join(XNOR_MODES), mode))
+    return mode
+
+
+def honour_xnor(xnor):
+    """The generator flag for a conv call of the CUDA-named module: True only in cuda_ref mode.  In the default
+    mode an xnor=True argument is accepted and not honoured; that is said once per process."""
+    global _warned_xnor_ignored
+    if not xnor:
+        return False
+    if xnor_mode() == "cuda_ref":
+        return True
+    if not _warned_xnor_ignored:
+        _warned_xnor_ignored = True
+        warnings.warn("sc_extension_cuda: xnor=True is accepted but not honoured: bit streams follow the reference's CPU "
+                      "extension (XOR-feedback LFSR).  Set REXSC_XNOR_MODE=cuda_ref for the CUDA extension's XNOR generator.",
+                      RuntimeWarning, stacklevel=3)
+    return False
 
 
 def _require_cuda(*tensors):
@@ -57,7 +87,7 @@ def _empty_out(shape, dtype, device, channels_last):
 
 
 def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
-              want_split=True, want_diff=False):
+              want_split=True, want_diff=False, xnor=False):
     """SC conv2d on the HIP path.  padding=(p0,p1): p0 pads the LAST axis, p1 axis 2, as the
     reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2."""
     _require_cuda(x, w)
@@ -70,7 +100,7 @@ def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_con
     O, _, KH, KW = wc.shape
     d = _lib.ConvDesc(N, C, H, W, O, KH, KW, int(padding[1]), int(padding[0]), int(stride[0]), int(stride[1]),
                       int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
-                      int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w))
+                      int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w), int(bool(xnor)))
     L = _lib.lib()
     with torch.cuda.device(x.device):
         Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1

@@ -36,10 +36,14 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 // ---- LFSR ------------------------------------------------------------------------------------
 // Fibonacci LFSRs of 3..8 bits; taps per width as in the reference CPU extension
 // (sc_cpu.hpp:49-137): 3:{2,1} 4:{3,2} 5:{4,2} 6:{5,4} 7:{6,5} 8:{7,5,4,3}.
-// acc != 0 splices the zero state into the cycle (1 -> 0 -> 2), sc_cpu.hpp:54-64.
+// Flavours (the `acc` argument): 0 plain; 1 ("_acc") splices the zero state into the cycle
+// (1 -> 0 -> 2), sc_cpu.hpp:54-64; 2 XNOR feedback, the generator the reference's CUDA conv kernels
+// select with xnor = true (sc_device.cuh:108-286): the complemented feedback bit is shifted in, the
+// cycle runs over 0 .. 2^lb-2 and the all-ones state is its fixed point.
+enum { LFSR_PLAIN = 0, LFSR_ACC = 1, LFSR_XNOR = 2 };
 __host__ __device__ inline int lfsr_step(int lb, int acc, int v)
 {
-    if (acc) {
+    if (acc == LFSR_ACC) {
         if (v == 1) return 0;
         if (v == 0) return 2;
     }
@@ -52,6 +56,7 @@ __host__ __device__ inline int lfsr_step(int lb, int acc, int v)
     case 7: fb = ((v >> 6) ^ (v >> 5)) & 1; break;
     default: fb = ((v >> 7) ^ (v >> 5) ^ (v >> 4) ^ (v >> 3)) & 1; break;
     }
+    if (acc == LFSR_XNOR) fb = 1 - fb;
     return fb + 2 * (v & ((1 << (lb - 1)) - 1));
 }
 
@@ -82,8 +87,9 @@ struct SeqTable {
     uint8_t seq[SEQ_LEN];
     uint8_t inv[256];
 };
-// table index for (lb in 3..8, acc in 0..1)
-__host__ __device__ inline int seq_index(int lb, int acc) { return (lb - 3) * 2 + acc; }
+// table index for (lb in 3..8, flavour in 0..2)
+constexpr int N_SEQ_TABLES = 18;
+__host__ __device__ inline int seq_index(int lb, int acc) { return (lb - 3) * 3 + acc; }
 
 // Device address of the per-device sequence tables (built on first use).
 int get_seq_tables(const SeqTable **tables, hipStream_t stream);
@@ -93,8 +99,9 @@ int get_seq_tables(const SeqTable **tables, hipStream_t stream);
 // cycle cyc(s) = (s / slot_div) * slot_mul + (s % slot_mod): activations use
 // (g*g, g, g) and weights (g, 1, 1) for gen_config g (sc_conv.cpp:127-130, 195-197).
 struct GenParams {
-    int lb, acc, period;             // LFSR width, flavour, 2^lb-1 (or 2^lb for acc)
-    int seed_mod;                    // 2^lb - 1: seeds are (index % seed_mod) + 1
+    int lb, acc, period;             // LFSR width, flavour (LFSR_*), cycle length: 2^lb-1 (2^lb for LFSR_ACC)
+    int seed_mod;                    // 2^lb - 1: seeds are (index % seed_mod) + seed_off
+    int seed_off;                    // 1; 0 for LFSR_XNOR, whose cycle includes state 0 (sc_cuda_conv.cu:55-56,139)
     int scale;                       // S: float operands are multiplied by S
     int n_slots;                     // slots to generate
     int slot_div, slot_mul, slot_mod;

@@ -64,8 +64,9 @@ int fill_gen(GenParams &g, int lb, int acc, int scale, int n_slots, int div, int
              int lwait, int bit_length)
 {
     g.lb = lb; g.acc = acc;
-    g.period = acc ? (1 << lb) : (1 << lb) - 1;
+    g.period = acc == LFSR_ACC ? (1 << lb) : (1 << lb) - 1;
     g.seed_mod = (1 << lb) - 1;
+    g.seed_off = acc == LFSR_XNOR ? 0 : 1;
     g.scale = scale;
     g.n_slots = n_slots;
     g.slot_div = div; g.slot_mul = mul; g.slot_mod = mod;
@@ -84,7 +85,7 @@ int fill_gen(GenParams &g, int lb, int acc, int scale, int n_slots, int div, int
 // of B pixels is the batch, 1x1 kernel).
 int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int pad_h, int pad_w, int s0, int s1,
               int bit_length, int lfsr_length, int gen_config, int bin_config, int tw, int lw, int lwait,
-              int act_cl, int w_cl, bool linear)
+              int act_cl, int w_cl, bool linear, bool xnor)
 {
     memset(&pl, 0, sizeof(pl));
     REXSC_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && O > 0 && KH > 0 && KW > 0, "non-positive dimension");
@@ -123,7 +124,13 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     const int ZC = pl.ZC, ZG = ceil_div(Z, ZC);
     const int OT = sc_compute_tile_ot();
     const int O_pad = (int)align_up((size_t)O, (size_t)OT);
-    const int acc = (!linear && g == 2) ? 1 : 0;
+    // CPU-extension rule: the and_2 generator steps the zero-including LFSR (sc_conv.cpp:365-425).  The CUDA
+    // kernels have no such variant: with xnor they step the XNOR LFSR for every gen_config, seeds lowered by
+    // one (sc_cuda_conv.cu:28,55-56,139), and keep seeds and operands in int8 (sc_cuda_conv.cu:37-40), which
+    // leaves 8-bit LFSRs without a meaningful result.
+    REXSC_CHECK_ARG(!(xnor && linear), "linear: the reference's linear kernels have no XNOR generator");
+    REXSC_CHECK_ARG(!(xnor && lb == 8), "xnor generator: 8-bit LFSRs are not supported (the CUDA reference keeps states in int8)");
+    const int acc = xnor ? LFSR_XNOR : ((!linear && g == 2) ? LFSR_ACC : LFSR_PLAIN);
     int rc = fill_gen(pl.gen_act, lb, acc, scale, n_slots, g * g, g, g, tw, lw, lwait, bit_length);
     if (rc) return rc;
     rc = fill_gen(pl.gen_w, lb, acc, scale, n_slots, g, 1, 1, tw, lw, lwait, bit_length);
@@ -226,7 +233,7 @@ int plan_conv(ScPlan &pl, const rexsc_conv_desc *d)
     REXSC_CHECK_ARG(d != nullptr, "null descriptor");
     return make_plan(pl, d->N, d->C, d->H, d->W, d->O, d->KH, d->KW, d->pad_h, d->pad_w, d->stride_h, d->stride_w,
                      d->bit_length, d->lfsr_length, d->gen_config, d->bin_config, d->total_width, d->load_width,
-                     d->load_wait, d->act_channels_last != 0, d->weight_channels_last != 0, false);
+                     d->load_wait, d->act_channels_last != 0, d->weight_channels_last != 0, false, d->xnor != 0);
 }
 
 int plan_linear(ScPlan &pl, const rexsc_linear_desc *d)
@@ -234,7 +241,7 @@ int plan_linear(ScPlan &pl, const rexsc_linear_desc *d)
     REXSC_CHECK_ARG(d != nullptr, "null descriptor");
     // batch rows become the pixels of a single 1 x B "image" in channels-last order
     int rc = make_plan(pl, 1, d->C, 1, d->B, d->O, 1, 1, 0, 0, 1, 1, d->bit_length, d->lfsr_length, d->gen_config,
-                       d->bin_config, d->total_width, d->load_width, d->load_wait, 1, 0, true);
+                       d->bin_config, d->total_width, d->load_width, d->load_wait, 1, 0, true, false);
     if (rc) return rc;
     if (pl.wide && !(pl.ZC == 4 || pl.ZC == 8)) {
         set_error("linear: internal planning error (wide accumulation with chunk width %d)", pl.ZC);

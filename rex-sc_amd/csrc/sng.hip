@@ -22,16 +22,16 @@
 namespace rexsc {
 
 // ---- sequence tables -------------------------------------------------------------------------
-static __device__ SeqTable g_seq_tables[12];
+static __device__ SeqTable g_seq_tables[N_SEQ_TABLES];
 
 __global__ void build_seq_tables_kernel()
 {
     int idx = threadIdx.x;
-    if (idx >= 12) return;
-    int lb = idx / 2 + 3, acc = idx % 2;
-    int period = acc ? (1 << lb) : (1 << lb) - 1;
+    if (idx >= N_SEQ_TABLES) return;
+    int lb = idx / 3 + 3, acc = idx % 3;
+    int period = acc == LFSR_ACC ? (1 << lb) : (1 << lb) - 1;
     SeqTable &t = g_seq_tables[idx];
-    int v = 1;
+    int v = acc == LFSR_XNOR ? 0 : 1; // a state on the cycle (the plain LFSR never reaches 0, the XNOR one never all-ones)
     for (int i = 0; i < 256; i++) t.inv[i] = 0;
     for (int i = 0; i < SEQ_LEN; i++) {
         t.seq[i] = (uint8_t)v;
@@ -238,7 +238,7 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
                 if (cl < CCH) v = s_q[cl * QPITCH + j];
                 int sd = cmod[h] + pmod;
                 if (sd >= gp.seed_mod) sd -= gp.seed_mod;
-                const int pos = s_inv[sd + 1] + 1; // state of cycle t is seq[pos + t]
+                const int pos = s_inv[sd + gp.seed_off] + 1; // state of cycle t is seq[pos + t]
                 uint32_t lo, hi;
                 gen_slots32(s_seq, pos, v, gp, s0, ns, lo, hi);
                 if (lane < ns) {
@@ -307,7 +307,7 @@ __device__ __forceinline__ void build_state_planes(const ActTableJob &job, const
         const int ch = z * 32 + cc;
         int sd = ((ch % gp.seed_mod) * cmul) % gp.seed_mod + pm;
         if (sd >= gp.seed_mod) sd -= gp.seed_mod;
-        const int pos = s_inv[sd + 1] + 1;
+        const int pos = s_inv[sd + gp.seed_off] + 1;
         if (job.shift) {
             int idx = pos + s - (gp.lb - 1); // cycle s - (lb - 1); the sequence has period gp.period
             if (idx < 0) idx += gp.period;
@@ -512,7 +512,7 @@ static ActTableJob act_table_job(uint32_t *T, const ActGeom &geo, const GenParam
     job.PM = geo.seed_pmul % gp.seed_mod == 0 ? 1 : gp.seed_mod;
     job.pitch = job.PM == 1 ? 1 : (1 << gp.lb);
     job.seed_cmul = geo.seed_cmul;
-    job.shift = (!gp.acc && gp.slot_div == 1 && gp.slot_mul == 1 && gp.slot_mod == 1) ? 1 : 0;
+    job.shift = (gp.acc != LFSR_ACC && gp.slot_div == 1 && gp.slot_mul == 1 && gp.slot_mod == 1) ? 1 : 0;
     job.n_tau = gp.n_slots + gp.lb - 1;
     return job;
 }
@@ -665,7 +665,7 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
                     const int h = combo % HALVES, kx = combo / HALVES;
                     const long c = (long)zg * CCH + h * 64 + lane;
                     const int sd = (int)((13L + c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
-                    s_pos[cl * 64 + lane] = s_inv[sd + 1];
+                    s_pos[cl * 64 + lane] = s_inv[sd + gp.seed_off];
                 }
                 __syncthreads();
             }

@@ -2,8 +2,9 @@
 
 Same function names, positional arguments and return conventions; the work runs on the HIP
 kernels of librexsc.so.  Arithmetic follows the reference's CPU extension, which the
-bit-exactness contract is defined against (in particular `xnor` is accepted and ignored, as
-sc_conv.cpp does).
+bit-exactness contract is defined against: by default `xnor` is accepted and ignored, as
+sc_conv.cpp does.  With REXSC_XNOR_MODE=cuda_ref in the environment the conv op honours it the
+way the reference's CUDA kernels do (XNOR-feedback LFSR, sc_cuda_conv.cu:28,55-56,139).
 """
 import _ops
 
@@ -12,7 +13,7 @@ def conv2d_generic_general_split_acc(input, weight, bit_length, lfsr_length, z_u
                                      bin_config, gen_config, xnor, mux):
     """[pos, neg] int16 [N,O,Ho,Wo]; channels_last iff the input is (sc_cuda.cpp:87-99)."""
     pos, neg, _ = _ops.sc_conv2d(input, weight, bit_length, lfsr_length, padding, stride, prog_load, bin_config,
-                                 gen_config, want_split=True)
+                                 gen_config, want_split=True, xnor=_ops.honour_xnor(xnor))
     return [pos, neg]
 
 
@@ -20,7 +21,7 @@ def conv2d_generic_general_acc(input, weight, bit_length, lfsr_length, z_units, 
                                bin_config, gen_config, xnor, mux):
     """pos - neg, int16 (sc_cuda.cpp:73-85)."""
     _, _, diff = _ops.sc_conv2d(input, weight, bit_length, lfsr_length, padding, stride, prog_load, bin_config,
-                                gen_config, want_split=False, want_diff=True)
+                                gen_config, want_split=False, want_diff=True, xnor=_ops.honour_xnor(xnor))
     return diff
 
 

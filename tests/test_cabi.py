@@ -91,7 +91,8 @@ def test_product_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f), encoding="utf-8", errors="replace").read()
                 for n, line in enumerate(text.splitlines(), 1):
-                    if pat.search(line) and "cpu_oracle" not in line:
+                    # the two names of the xnor modes are not references to the oracle directory
+                    if pat.search(line.replace("cpu_oracle", "").replace("cuda_ref", "")):
                         offenders.append("%s:%d: %s" % (os.path.relpath(os.path.join(dirpath, f), root), n, line.strip()))
     assert not offenders, "\n".join(offenders)
     extra = open(os.path.join(root, "bench_extra.py")).read()

@@ -234,3 +234,63 @@ def test_fixed_random_vs_oracle(cfg):
     want = orc.conv2d_saturate(x, w, add, pin, pout, pad, stride)
     assert out.shape == want.shape and np.abs(want).max() > 0
     assert np.array_equal(out.cpu().numpy(), want)
+
+
+# ---- REXSC_XNOR_MODE=cuda_ref: the generators of the reference's CUDA conv kernels ---------------------------
+XNOR_CONV = [
+    # N, C, H, W, O, K, stride, L, lfsr_length, bin_config, gen, cl_act, cl_w
+    (2, 64, 14, 14, 48, 3, 1, 32, -1, 1, 1, True, False),
+    (2, 64, 56, 56, 64, 3, 1, 32, -1, 1, 1, True, False),    # ResNet-18 layer1 shape: bit-sliced generator, shift table
+    (1, 33, 9, 11, 20, 3, 2, 64, -1, 2, 1, False, True),
+    (2, 3, 32, 32, 32, 3, 1, 64, -1, 2, 1, False, False),
+    (1, 40, 8, 8, 24, 5, 1, 16, -1, 0, 2, False, False),     # and_2 with the XNOR LFSR (no "_acc" variant on CUDA)
+    (1, 16, 6, 6, 8, 1, 1, 32, 7, 3, 2, True, False),
+    (1, 8, 5, 5, 4, 3, 1, 8, -1, 1, 1, False, False),
+    (1, 512, 7, 7, 64, 3, 1, 128, -1, 1, 1, True, False),
+]
+
+
+@pytest.mark.parametrize("sng_mode", ["0", "1", "2"])
+@pytest.mark.parametrize("cfg", XNOR_CONV, ids=lambda c: "_".join(str(v) for v in c))
+def test_conv_cuda_xnor_mode_vs_oracle(cfg, sng_mode, monkeypatch):
+    import sc_extension
+    import sc_extension_cuda
+    N, C, H, W, O, K, stride, L, lfsr, bc, gen, cla, clw = cfg
+    print("conv cuda_xnor", cfg, "sng mode", sng_mode, flush=True)
+    monkeypatch.setenv("REXSC_XNOR_MODE", "cuda_ref")
+    monkeypatch.setenv("REXSC_SNG_MODE", sng_mode)
+    rng = np.random.default_rng(hash(cfg) & 0xFFFF)
+    S = (1 << lfsr) if lfsr > 0 else L
+    dens = min(1.0, 96.0 / (C * K * K) + 0.02)
+    x = (rng.integers(0, S, size=(N, C, H, W)) / S * (rng.uniform(size=(N, C, H, W)) < dens)).astype(np.float32)
+    w = (rng.integers(-S + 1, S, size=(O, C, K, K)) / S * (rng.uniform(size=(O, C, K, K)) < dens)).astype(np.float32)
+    pad = (K // 2, K // 2)
+    args = (_dev(x, cla), _dev(w, clw), L, lfsr, 16, pad, (stride, stride), (7, 8, 1), bc, gen)
+    pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(*args, True, False)
+    opos, oneg = orc.conv2d_generic_general_split(x, w, L, lfsr, 16, pad, (stride, stride), (7, 8, 1), bc, gen,
+                                                  channels_last_activation=cla, channels_last_weight=clw, cuda_xnor=True)
+    assert opos.max() > 0
+    assert np.array_equal(pos.cpu().numpy(), opos) and np.array_equal(neg.cpu().numpy(), oneg)
+    # xnor=False in the same mode, and the CPU-named module in any mode, keep the CPU extension's generator
+    cpos, cneg = orc.conv2d_generic_general_split(x, w, L, lfsr, 16, pad, (stride, stride), (7, 8, 1), bc, gen,
+                                                  channels_last_activation=cla, channels_last_weight=clw)
+    assert not np.array_equal(cpos, opos)
+    p0, n0 = sc_extension_cuda.conv2d_generic_general_split_acc(*args, False, False)
+    assert np.array_equal(p0.cpu().numpy(), cpos) and np.array_equal(n0.cpu().numpy(), cneg)
+    d0 = sc_extension.conv2d_generic_general(*args, True, False)
+    assert np.array_equal(d0.cpu().numpy(), (cpos.astype(np.int32) - cneg).astype(np.int16))
+
+
+def test_cuda_xnor_mode_rejections_and_default(monkeypatch):
+    import _ops
+    import sc_extension_cuda
+    x = torch.rand(1, 8, 6, 6, device="cuda")
+    w = torch.rand(4, 8, 3, 3, device="cuda")
+    monkeypatch.delenv("REXSC_XNOR_MODE", raising=False)
+    assert _ops.xnor_mode() == "cpu_oracle"
+    monkeypatch.setenv("REXSC_XNOR_MODE", "cuda_ref")
+    with pytest.raises(RuntimeError, match="8-bit"):
+        sc_extension_cuda.conv2d_generic_general_split_acc(x, w, 256, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1, True, False)
+    monkeypatch.setenv("REXSC_XNOR_MODE", "something")
+    with pytest.raises(RuntimeError, match="REXSC_XNOR_MODE"):
+        sc_extension_cuda.conv2d_generic_general_split_acc(x, w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1, True, False)

@@ -228,3 +228,99 @@ def test_linear_slot_interleave_brute_force(g, bc):
                 exp_n[b, o] += (cn >= n_sat) if bc < 0 else min(cn, n_sat)
     pos, neg = orc.linear_generic_general(x, w, (7, 8, 1), L, -1, bc, g)
     assert np.array_equal(pos, exp_p) and np.array_equal(neg, exp_n)
+
+
+# ---- the XNOR generator of the reference's CUDA conv kernels (no CUDA build or fixture exists) --------------
+@pytest.mark.parametrize("lb", [3, 4, 5, 6, 7, 8])
+def test_xnor_lfsr_cycle_and_complement_relation(lb):
+    """sc_device.cuh:108-286: the XNOR LFSR runs over 0 .. 2^lb-2 with period 2^lb-1 and all-ones as its fixed
+    point; every tap set has an even number of taps, so it is the bitwise complement of the plain LFSR:
+    xnor_step(~s) == ~xor_step(s)."""
+    full = (1 << lb) - 1
+    seen, v = [], 0
+    for _ in range(full):
+        seen.append(v)
+        v = orc.lfsr_step(lb, 2, v)
+    assert v == 0 and sorted(seen) == list(range(full))
+    assert orc.lfsr_step(lb, 2, full) == full
+    for s in range(full + 1):
+        assert orc.lfsr_step(lb, 2, full ^ s) == full ^ orc.lfsr_step(lb, 0, s)
+
+
+def _cuda_xnor_step(lb, v):
+    """The reference's own arithmetic, d_lfsr_N_xnor (sc_device.cuh:108,147,172,197,224,244)."""
+    if lb == 3:
+        return 1 - ((v // 4) + (v // 2) % 2) % 2 + 2 * (v % 4)
+    if lb == 4:
+        return 1 - ((v // 8) + (v // 4) % 2) % 2 + 2 * (v % 8)
+    if lb == 5:
+        return 1 - ((v // 16) + (v // 4) % 2) % 2 + 2 * (v % 16)
+    if lb == 6:
+        return 1 - ((v // 32) + (v // 16) % 2) % 2 + 2 * (v % 32)
+    if lb == 7:
+        return 1 - ((v // 64) + (v // 32) % 2) % 2 + 2 * (v % 64)
+    return 1 - ((v // 128) + (v // 32) % 2 + (v // 16) % 2 + (v // 8) % 2) % 2 + 2 * (v % 128)
+
+
+@pytest.mark.parametrize("L,gen,bc", [(8, 1, 0), (16, 1, 1), (32, 1, 1), (32, 2, 1), (64, 1, 2), (16, 2, 0)])
+def test_cuda_xnor_conv_brute_force(L, gen, bc):
+    """The oracle's cuda_xnor mode against a per-bit Python model written from sc_cuda_conv.cu:3-166 (seeds
+    (13 + c*KH*KW + ky*KW + kx) % P + 1 - 1 and (c*Hp*Wp + y*Wp + x) % P + 1 - 1, state stepped before the
+    compare, the same LFSR for gen_config 2, slot interleave :90-93,160-162) and the per-slot saturating sum."""
+    rng = np.random.default_rng(L + gen)
+    N, C, H, W, O, K = 1, 5, 4, 5, 3, 3
+    lb = orc.lfsr_bits(L)
+    P = (1 << lb) - 1
+    for s in range(P + 1):  # the step the model uses is the reference's own formula
+        assert _cuda_xnor_step(lb, s) == orc.lfsr_step(lb, 2, s)
+    x = (rng.integers(0, L, size=(N, C, H, W)) / L).astype(np.float32)
+    w = (rng.integers(-L + 1, L, size=(O, C, K, K)) / L).astype(np.float32)
+    got_p, got_n = orc.conv2d_generic_general_split(x, w, L, -1, 16, (1, 1), (1, 1), (7, 8, 1), bc, gen, cuda_xnor=True)
+    xq = np.pad(orc.quantize_sc(x, L, 0), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    wq = (orc.quantize_sc(w, L, 0), orc.quantize_sc(w, L, 1))
+    Hp, Wp, T = H + 2, W + 2, L * gen
+
+    def stream(value, seed):
+        bits, st = [], seed
+        for _ in range(L):
+            st = _cuda_xnor_step(lb, st)
+            bits.append(int(value > st))
+        return bits
+
+    a_slots = np.zeros((T, C, Hp, Wp), np.int64)
+    for c in range(C):
+        for y in range(Hp):
+            for xx in range(Wp):
+                b = stream(xq[0, c, y, xx], (c * Hp * Wp + y * Wp + xx) % P + 1 - 1)
+                for t in range(L):
+                    for j in range(gen):
+                        a_slots[(t // gen) * gen * gen + j * gen + t % gen, c, y, xx] = b[t]
+    w_slots = np.zeros((2, T, O, C, K, K), np.int64)
+    for pol in range(2):
+        for o in range(O):
+            for c in range(C):
+                for ky in range(K):
+                    for kx in range(K):
+                        b = stream(wq[pol][o, c, ky, kx], (13 + c * K * K + ky * K + kx) % P + 1 - 1)
+                        for t in range(L):
+                            for j in range(gen):
+                                w_slots[pol, t * gen + j, o, c, ky, kx] = b[t]
+    n_sat = bc + 1
+    for pol, got in ((0, got_p), (1, got_n)):
+        want = np.zeros((N, O, H, W), np.int64)
+        for t in range(T):
+            cnt = F.conv2d(torch.from_numpy(a_slots[t][None].astype(np.float64)),
+                           torch.from_numpy(w_slots[pol, t].astype(np.float64))).numpy()
+            want += np.minimum(cnt.astype(np.int64), n_sat)
+        assert want.max() > 0
+        assert np.array_equal(got.astype(np.int64), want)
+    # and it is a different generator: the CPU-extension result differs
+    cpu_p, _ = orc.conv2d_generic_general_split(x, w, L, -1, 16, (1, 1), (1, 1), (7, 8, 1), bc, gen)
+    assert not np.array_equal(cpu_p, got_p)
+
+
+def test_cuda_xnor_refuses_8_bit_lfsrs():
+    x = np.zeros((1, 4, 4, 4), np.float32)
+    w = np.zeros((2, 4, 3, 3), np.float32)
+    with pytest.raises(ValueError):
+        orc.conv2d_generic_general_split(x, w, 256, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1, cuda_xnor=True)
