@@ -110,6 +110,18 @@ int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, const float *w,
                      int32_t *out_pos, int32_t *out_neg,
                      void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
 
+/* The reference's legacy pure-torch simulation `linear_generic` (utils_functional.py:955-1081 with the
+ * generators of :147-165, 254-272; generator 'lfsr', shared generators; what its Linear_Or layer runs,
+ * utils_class.py:183-208) on the same kernels: operands q = ceil(float16(x * L)) with activations
+ * unclamped and weight parts clamped to weight_clamp (the function's `prec - 1`: 127), seeds
+ * (67 + c) % P + 1 / (37 + c) % P + 1 for the positive / negative weight part and c % P + 1 for
+ * activations, P = L - 1.  bin_config 0 is its forward 'full_or' (per-cycle OR), 51200 its 'full_bin'.
+ * bit_length 8..128, lfsr_length <= 0, gen_config 1, no progressive loading.  Outputs are the per-output
+ * sums over the L cycles (the function returns them divided by L).  Workspace: rexsc_linear_workspace_bytes. */
+int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp, const float *x, const float *w,
+                        int32_t *out_pos, int32_t *out_neg,
+                        void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
 /* ---- OR-n pointwise activation ---------------------------------------------------------
  * y = n - exp(-x) * sum_{i<n} (n-i) x^i / i!  for n = 1..4, float32.
  * Replaces sc_extension_cuda.or_approx_n_forward_acc / _backward_acc (sc_cuda_pw.cu:708-811);

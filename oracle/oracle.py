@@ -12,7 +12,8 @@ are NOT used: the reference works in float32 tensors, and so does this).
 Pinning: the conv / linear / fixed-conv functions against tests/golden/ref_cpu_ext.npz (hand-picked
 cases) and ref_cpu_ext_random.npz (96 seeded random configurations), both written by the
 reference's compiled CPU extension; compute_bias_std_coef against tests/golden/ref_calib.npz
-(written by the reference's own Python function); the scalar float functions (OR-n, bias/noise,
+(written by the reference's own Python function); linear_generic_legacy against tests/golden/ref_linear_legacy.npz
+(likewise); the scalar float functions (OR-n, bias/noise,
 quantise) against closed forms in tests/test_oracle_invariants.py.
 
 Parity unpinned: the linear op with an 8-bit LFSR (256-bit streams or lfsr_length 8).  The
@@ -285,3 +286,42 @@ def compute_bias_std_coef(or_n, a_bit, a_act, order):
         bias_coef = np.linalg.lstsq(A.astype(np.float64), bias_bins.astype(np.float64), rcond=None)[0].astype(np.float32)
     std_coef = np.linalg.lstsq(A.astype(np.float64), std_bins.astype(np.float64), rcond=None)[0].astype(np.float32)
     return bias_coef, std_coef
+
+
+def linear_generic_legacy(x, w, bit_length, forward="full_or", prec=128):
+    """The reference's legacy `linear_generic` (utils_functional.py:955-1081; generator 'lfsr', share=True) with
+    its generators (:147-165 lfsr_init, :254-272 lfsr_cont) -> float32 [B,O], pos - neg.
+
+    Restated cycle by cycle in numpy: operands are the float16-rounded products x*L (weights clamped to
+    prec-1 per polarity, activations unclamped; :980-995), LFSR states are integers stepped before the compare
+    (:1022), seeds c % P + 1 / (67 + c) % P + 1 / (37 + c) % P + 1 with P = L - 1 shared by all rows (:1000-1001),
+    per cycle sign(count) ('full_or') or count ('full_bin') (:1031-1036), mean over cycles rounded to float16
+    (compute_type, :28; :1067-1068).  Pinned by tests/golden/ref_linear_legacy.npz, written by the reference's own
+    function."""
+    x = np.asarray(x, np.float32)
+    w = np.asarray(w, np.float32)
+    L = int(bit_length)
+    lb = {8: 3, 16: 4, 32: 5, 64: 6, 128: 7, 256: 8}[L]
+    P = L - 1
+    bit_range = np.float32(prec - 1)
+    Lf = np.float32(L)
+    a = (x * Lf).astype(np.float16).astype(np.float32)
+    wp = np.clip(w * Lf, 0, bit_range).astype(np.float16).astype(np.float32)
+    wn = (-np.clip(w * Lf, -bit_range, 0)).astype(np.float16).astype(np.float32)
+    C = x.shape[1]
+    c = np.arange(C)
+    st_a, st_p, st_n = c % P + 1, (67 + c) % P + 1, (37 + c) % P + 1
+    step = np.vectorize(lambda v: lfsr_step(lb, 0, int(v)))
+    pos = np.zeros((x.shape[0], w.shape[0]), np.float64)
+    neg = np.zeros_like(pos)
+    for _ in range(L):
+        st_a, st_p, st_n = step(st_a), step(st_p), step(st_n)
+        ab = (a > st_a).astype(np.float64)
+        cp = ab @ (wp > st_p).astype(np.float64).T
+        cn = ab @ (wn > st_n).astype(np.float64).T
+        if forward == "full_or":
+            cp, cn = np.sign(cp), np.sign(cn)
+        pos += cp
+        neg += cn
+    mean = lambda t: (t / L).astype(np.float32).astype(np.float16).astype(np.float32)
+    return mean(pos) - mean(neg)

@@ -150,6 +150,35 @@ def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config):
     return pos, neg
 
 
+def sc_linear_legacy(x, w, bit_length, bin_config, weight_clamp=127):
+    """The reference's legacy `linear_generic` simulation (utils_functional.py:955-1081, generator 'lfsr',
+    shared generators) on the HIP kernels -> (pos, neg) int32 [B,O]: per-output sums over the bit_length cycles."""
+    _require_cuda(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.size(1) != w.size(1):
+        raise RuntimeError("linear: expected input [B,C] and weight [O,C], got %s and %s"
+                           % (tuple(x.shape), tuple(w.shape)))
+    xc = x.detach().float().contiguous()
+    wc = w.detach().float().contiguous()
+    B, C = xc.shape
+    O = wc.shape[0]
+    d = _lib.LinearDesc(B, C, O, int(bit_length), -1, 1, int(bin_config), 7, 8, 1)
+    L = _lib.lib()
+    if B == 0:
+        return (torch.empty((0, O), dtype=torch.int32, device=x.device),
+                torch.empty((0, O), dtype=torch.int32, device=x.device))
+    with torch.cuda.device(x.device):
+        ws_bytes = L.rexsc_linear_workspace_bytes(ctypes.byref(d))
+        if ws_bytes == 0:
+            _lib.check(-1, "rexsc_linear_legacy (planning)")
+        pos = torch.empty((B, O), dtype=torch.int32, device=x.device)
+        neg = torch.empty((B, O), dtype=torch.int32, device=x.device)
+        ws = _workspace(ws_bytes, x.device)
+        rc = L.rexsc_linear_legacy(ctypes.byref(d), int(weight_clamp), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws),
+                                   ws.numel(), _stream())
+        _lib.check(rc, "rexsc_linear_legacy")
+    return pos, neg
+
+
 def fixed_conv2d(x, w, add_config, precision_in, precision_out, padding, stride):
     _require_cuda(x, w)
     if x.dim() != 4 or w.dim() != 4 or x.size(1) != w.size(1):

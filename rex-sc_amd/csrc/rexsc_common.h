@@ -107,6 +107,14 @@ struct GenParams {
     int slot_div, slot_mul, slot_mod;
     int total_width, load_width, load_wait; // progressive loading
     int prog;                        // 0 when the truncation shift is 0 for every cycle
+    int seed_add;                    // constant added to the seed index: 13 for weights (sc_cpu.hpp:10-11), 0 for activations
+    // Operand quantisation: q = ceil(clamp(x * scale, 0, clamp_hi)), clamp_hi = scale - 1 (sc_conv.cpp:318-320).
+    // legacy != 0 is the rule of the reference's pure-torch simulation `linear_generic`
+    // (utils_functional.py:980-995, 1022-1024): the product is rounded to binary16 first, clamp_hi is set by the
+    // caller and may reach `scale`, a value above every LFSR state ("always one").
+    int legacy;
+    float clamp_hi;
+    float sign;                      // weights only: operand multiplied by +1 / -1 before the split into polarities
 };
 
 __host__ __device__ inline int slot_cycle(const GenParams &g, int s)

@@ -72,6 +72,7 @@ int fill_gen(GenParams &g, int lb, int acc, int scale, int n_slots, int div, int
     g.slot_div = div; g.slot_mul = mul; g.slot_mod = mod;
     g.total_width = tw; g.load_width = lw; g.load_wait = lwait;
     g.prog = 0;
+    g.seed_add = 0; g.legacy = 0; g.clamp_hi = (float)(scale - 1); g.sign = 1.f;
     REXSC_CHECK_ARG(lwait >= 1, "prog_load: load_wait must be >= 1 (got %d)", lwait);
     for (int t = 0; t < bit_length; t++) {
         const int sh = prog_shift(g, t);
@@ -135,6 +136,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     if (rc) return rc;
     rc = fill_gen(pl.gen_w, lb, acc, scale, n_slots, g, 1, 1, tw, lw, lwait, bit_length);
     if (rc) return rc;
+    pl.gen_w.seed_add = 13; // POS_SEED == NEG_SEED (sc_cpu.hpp:10-11)
 
     // batch chunking
     const size_t words_per_image_slot = (size_t)ZG * Hp * Wp * ZC;
@@ -432,4 +434,55 @@ extern "C" int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, cons
     rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, stream);
     if (rc) return rc;
     return sc_finalize_i32(part, pl.cp, pl.wide, out_pos, out_neg, stream);
+}
+
+// The reference's legacy pure-torch simulation `linear_generic` (utils_functional.py:955-1081; generator 'lfsr',
+// shared generators): the same AND / popcount / per-cycle rule as the extension's linear op, with
+//   * operands q = ceil(float16(x * L)), activations unclamped (anything >= L is "always one"), weight parts
+//     clamped to weight_clamp (the function's `prec - 1`, 127 by default) -- the simulation compares the
+//     float16 products with integer LFSR states, and v > s for an integer s is ceil(v) > s;
+//   * seeds (67 + c) % P + 1 for the positive and (37 + c) % P + 1 for the negative weight part, c % P + 1
+//     for activations (utils_functional.py:147-165).
+// Two passes over one set of activation streams, one per weight polarity (each with its own seeds).
+extern "C" int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp, const float *x, const float *w,
+                                   int32_t *out_pos, int32_t *out_neg, void *workspace, size_t workspace_bytes,
+                                   rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_linear(pl, d);
+    if (rc) return rc;
+    REXSC_CHECK_ARG(x && w && out_pos && out_neg, "null pointer");
+    REXSC_CHECK_ARG(d->lfsr_length <= 0 && d->gen_config == 1 && d->bit_length >= 8 && d->bit_length <= 128,
+                    "legacy linear: stream lengths 8..128 with the LFSR of that length and gen_config 1 only");
+    REXSC_CHECK_ARG(d->total_width == 7 && d->load_width == 8 && d->load_wait == 1, "legacy linear: no progressive loading");
+    REXSC_CHECK_ARG(weight_clamp >= 1, "legacy linear: weight_clamp must be positive");
+    if (!workspace || workspace_bytes < pl.total) {
+        set_error("legacy linear: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
+        return REXSC_ERR_WORKSPACE;
+    }
+    REXSC_CHECK_ARG(pl.tuned, "linear: no kernel instance for chunk width %d", pl.ZC);
+    uint8_t *ws = (uint8_t *)workspace;
+    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
+    uint32_t *A = (uint32_t *)(ws + pl.off_a);
+    uint32_t *part = (uint32_t *)(ws + pl.off_part);
+    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
+    const float L = (float)d->bit_length;
+    pl.gen_act.legacy = 1; pl.gen_act.clamp_hi = L;
+    pl.gen_w.legacy = 1; pl.gen_w.clamp_hi = weight_clamp < d->bit_length ? (float)weight_clamp : L;
+    for (int pol = 0; pol < 2; pol++) {
+        pl.gen_w.seed_add = pol == 0 ? 67 : 37;
+        pl.gen_w.sign = pol == 0 ? 1.f : -1.f; // pass 1 streams -w: its positive part is w's negative part
+        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, pol == 0 ? tab_a : nullptr, &pl.ag, &pl.gen_act, stream);
+        if (rc) return rc;
+        if (pol == 0) {
+            rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
+            if (rc) return rc;
+        }
+        rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, stream);
+        if (rc) return rc;
+        rc = sc_finalize_i32(part, pl.cp, pl.wide, pol == 0 ? out_pos : out_neg, nullptr, stream);
+        if (rc) return rc;
+    }
+    return REXSC_OK;
 }

@@ -67,10 +67,17 @@ int get_seq_tables(const SeqTable **tables, hipStream_t stream)
 }
 
 // ---- helpers -------------------------------------------------------------------------------
-__device__ __forceinline__ int quant_ceil_pos(float v, float S)
-{   // ceil(clamp(v*S, 0, S-1))
+// x * S as the generator sees it: exact float32 product, rounded to binary16 in legacy mode
+__device__ __forceinline__ float scaled_operand(float v, float S, int legacy)
+{
     float t = v * S;
-    t = fminf(fmaxf(t, 0.f), S - 1.f);
+    if (legacy) t = (float)(_Float16)t; // round to nearest even, as a tensor cast to float16 does
+    return t;
+}
+__device__ __forceinline__ int quant_ceil_pos(float v, float S, float hi, int legacy)
+{   // ceil(clamp(v*S, 0, hi))
+    float t = scaled_operand(v, S, legacy);
+    t = fminf(fmaxf(t, 0.f), hi);
     return (int)ceilf(t);
 }
 __device__ __forceinline__ void load_tables_to_lds(const SeqTable *tab, uint8_t *seq, uint8_t *inv)
@@ -187,7 +194,7 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
             v[k] = (inb && c < geo.C) ? x[(((long)n * geo.C + c) * geo.H + y) * geo.W + xx] : 0.f;
         }
 #pragma unroll
-        for (int k = 0; k < PER; k++) s_q[(wave + 4 * k) * QPITCH + lane] = (uint8_t)quant_ceil_pos(v[k], S);
+        for (int k = 0; k < PER; k++) s_q[(wave + 4 * k) * QPITCH + lane] = (uint8_t)quant_ceil_pos(v[k], S, gp.clamp_hi, gp.legacy);
     } else {
         // lane = channel, each wave takes 16 pixels
         constexpr int PIX = ACT_TILE / 4, PASS = (CCH + 63) / 64;
@@ -211,7 +218,7 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
 #pragma unroll
             for (int h = 0; h < PASS; h++) {
                 const int cl = h * 64 + lane;
-                if (cl < CCH) s_q[cl * QPITCH + wave + 4 * k] = (uint8_t)quant_ceil_pos(v[k][h], S);
+                if (cl < CCH) s_q[cl * QPITCH + wave + 4 * k] = (uint8_t)quant_ceil_pos(v[k][h], S, gp.clamp_hi, gp.legacy);
             }
     }
     __syncthreads();
@@ -364,19 +371,19 @@ __device__ __forceinline__ void values_to_planes(uint32_t (&R)[8])
     transpose_round<4, 0x0f0f0f0fu>(R[2], R[6]); transpose_round<4, 0x0f0f0f0fu>(R[3], R[7]);
 }
 
-// ceil(clamp(v*S, 0, S-1)) of channel c, deposited in its byte of the packed registers
+// ceil(clamp(v*S, 0, hi)) of channel c, deposited in its byte of the packed registers
 template <int C>
-__device__ __forceinline__ void pack_quantised(uint32_t (&R)[8], float v, float S)
+__device__ __forceinline__ void pack_quantised(uint32_t (&R)[8], float v, float S, float hi, int legacy)
 {
-    float t = v * S;
-    t = ceilf(fminf(fmaxf(t, 0.f), S - 1.f));
+    float t = scaled_operand(v, S, legacy);
+    t = ceilf(fminf(fmaxf(t, 0.f), hi));
     R[C & 7] = __builtin_amdgcn_cvt_pk_u8_f32(t, C >> 3, R[C & 7]);
 }
 template <int... C>
-__device__ __forceinline__ void pack_quantised_all(uint32_t (&R)[8], const float (&v)[32], float S,
+__device__ __forceinline__ void pack_quantised_all(uint32_t (&R)[8], const float (&v)[32], float S, float hi, int legacy,
                                                    std::integer_sequence<int, C...>)
 {
-    (pack_quantised<C>(R, v[C], S), ...);
+    (pack_quantised<C>(R, v[C], S, hi, legacy), ...);
 }
 
 template <int LB, bool PIXSEED, bool SHIFT>
@@ -425,12 +432,14 @@ __global__ __launch_bounds__(256) void sng_act_sliced_kernel(const float *__rest
 #pragma unroll
             for (int cc = 0; cc < 32; cc++) v[cc] = c0 + cc < geo.C ? src[cc * plane] : 0.f;
         }
-        pack_quantised_all(R, v, S, std::make_integer_sequence<int, 32>{});
+        pack_quantised_all(R, v, S, gp.clamp_hi, gp.legacy, std::make_integer_sequence<int, 32>{});
         values_to_planes(R);
     }
     uint32_t V[LB];
 #pragma unroll
     for (int k = 0; k < LB; k++) V[k] = R[k];
+    // legacy quantisation can reach 2^LB, one more than any LFSR state: those channels are always one
+    const uint32_t vtop = gp.legacy ? R[LB & 7] : 0u;
 
     constexpr int PITCH = PIXSEED ? (1 << LB) : 1; // words per table row
     const int pm = PIXSEED ? ((pp % gp.seed_mod) * (geo.seed_pmul % gp.seed_mod)) % gp.seed_mod : 0;
@@ -457,7 +466,7 @@ __global__ __launch_bounds__(256) void sng_act_sliced_kernel(const float *__rest
             for (int u = 0; u < U; u++) {
                 if (g0 + u < n_mine) {
                     const int first = gp.prog ? prog_shift(gp, s_begin + g0 + u) : 0;
-                    dst[(long)(g0 + u) * geo.slot_stride] = planes_greater<LB>(V, W, first);
+                    dst[(long)(g0 + u) * geo.slot_stride] = planes_greater<LB>(V, W, first) | vtop;
                 }
 #pragma unroll
                 for (int k = LB - 1; k > 0; k--) W[k] = W[k - 1];
@@ -484,7 +493,7 @@ __global__ __launch_bounds__(256) void sng_act_sliced_kernel(const float *__rest
             for (int u = 0; u < U; u++) {
                 if (g0 + u < n_mine) {
                     const int first = gp.prog ? prog_shift(gp, slot_cycle(gp, s_begin + g0 + u)) : 0;
-                    dst[(long)(g0 + u) * geo.slot_stride] = planes_greater<LB>(V, Sa[u], first);
+                    dst[(long)(g0 + u) * geo.slot_stride] = planes_greater<LB>(V, Sa[u], first) | vtop;
                 }
             }
 #pragma unroll
@@ -658,13 +667,13 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
         for (int combo0 = 0; combo0 < ncombo; combo0 += CCHUNK) {
             const int ncc = min(CCHUNK, ncombo - combo0);
             // cycle position of every channel's seed, lane = channel of the 64-channel half:
-            // seed (13 + c*KH*KW + ky*KW + kx) % seed_mod + 1  (sc_conv.cpp:80,92-93)
+            // seed (seed_add + c*KH*KW + ky*KW + kx) % seed_mod + seed_off, seed_add = 13  (sc_conv.cpp:80,92-93)
             if (s0 == 0 || ncombo > CCHUNK) {
                 for (int cl = wave; cl < ncc; cl += 4) {
                     const int combo = combo0 + cl;
                     const int h = combo % HALVES, kx = combo / HALVES;
                     const long c = (long)zg * CCH + h * 64 + lane;
-                    const int sd = (int)((13L + c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
+                    const int sd = (int)(((long)gp.seed_add + c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
                     s_pos[cl * 64 + lane] = s_inv[sd + gp.seed_off];
                 }
                 __syncthreads();
@@ -724,14 +733,14 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
 #pragma unroll
                 for (int i = 0; i < Q; i++) {
                     if (tq[i].ol >= wog) continue; // past the last task (wave-uniform)
-                    const float f = cur[i];
+                    const float f = cur[i] * gp.sign;
                     const int cl = tq[i].cl, ol = tq[i].ol;
                     const int combo = combo0 + cl;
                     const int h = combo % HALVES, kx = combo / HALVES;
                     // A weight feeds one polarity only (the other one quantises to 0): ballot the planes
                     // of the magnitude ceil(min(|f*S|, S-1)) and split them with the sign mask.  A NaN
                     // counts as negative, as it does in ceil(-clamp(f*S, 1-S, 0)).
-                    const uint32_t mag = (uint32_t)(int)ceilf(fminf(fabsf(f * S), S - 1.f));
+                    const uint32_t mag = (uint32_t)(int)ceilf(fminf(fabsf(scaled_operand(f, S, gp.legacy)), gp.clamp_hi));
                     const unsigned long long neg = __ballot(!(f >= 0.f));
                     uint32_t gt_p[NW], gt_n[NW];
 #pragma unroll
@@ -750,6 +759,16 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
                             const uint32_t dp = vkp ^ sk, dn = vkn ^ sk;
                             gt_p[wq] = (dp & vkp) | (~dp & gt_p[wq]);
                             gt_n[wq] = (dn & vkn) | (~dn & gt_n[wq]);
+                        }
+                    }
+                    if (gp.legacy) { // magnitudes of 2^LB (above every state): always one
+                        const unsigned long long m = __ballot((mag >> LB) & 1u);
+                        const unsigned long long mp = m & ~neg, mn = m & neg;
+#pragma unroll
+                        for (int wq = 0; wq < NW; wq++) {
+                            const bool hi = S64 ? wq == 1 : wsel != 0;
+                            gt_p[wq] |= hi ? (uint32_t)(mp >> 32) : (uint32_t)mp;
+                            gt_n[wq] |= hi ? (uint32_t)(mn >> 32) : (uint32_t)mn;
                         }
                     }
 #pragma unroll

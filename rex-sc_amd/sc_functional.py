@@ -556,3 +556,52 @@ def linear_generic_sc(activation, weight, **kwargs):
         pos_value.data = pos.to(activation.dtype) / bit_length
         neg_value.data = neg.to(activation.dtype) / bit_length
     return pos_value - neg_value
+
+
+def linear_or_approx(activation, weight, true_or=False):
+    """Float surrogate of OR accumulation for linear layers (utils_functional.py:600-608)."""
+    if true_or:
+        return 1 - torch.prod(1 - activation.unsqueeze(1) * weight, dim=-1)
+    return 1 - torch.exp(-F.linear(activation, weight))
+
+
+def linear_generic(activation, weight, **kwargs):
+    """The reference's legacy generic linear layer (utils_functional.py:955-1081), which its Linear_Or runs
+    (utils_class.py:183-208): a bit-by-bit simulation of the SC product in plain torch ops there, the same
+    numbers from the HIP kernels here (rexsc_linear_legacy).
+
+    bit_length, prec (128), share (True), generator, forward ('full_or' | 'full_bin') mean what they mean in the
+    reference.  Live configuration only: generator 'lfsr' with shared generators; the simulated true-random
+    generator, 'lfsr_split' and share=False are not built and raise.  The forward value is the SC result
+    (sum over the cycles / bit_length, the simulation's `.mean(0)`), gradients are those of the float surrogate
+    1 - exp(-x w_pos^T) - (1 - exp(-x w_neg^T)) ('full_or') or x w^T ('full_bin').  The reference's result tensor
+    ends up float16 (its compute_type, :28-29); the values here are the same numbers as float32 -- for 'full_bin'
+    after the float16 rounding its `.mean(0)` applies."""
+    bit_length = setvalue_default(kwargs, "bit_length", 128)
+    prec = setvalue_default(kwargs, "prec", 128)
+    share = setvalue_default(kwargs, "share", True)
+    generator = setvalue_default(kwargs, "generator", None)
+    forward = setvalue_default(kwargs, "forward", "full_or")
+    if forward not in ("full_or", "full_bin"):
+        raise ValueError("linear_generic: forward must be 'full_or' or 'full_bin' (got %r)" % (forward,))
+    if generator != "lfsr" or not share:
+        raise ValueError("linear_generic: only generator='lfsr' with share=True is built (got generator=%r, share=%r)"
+                         % (generator, share))
+    bit_range = prec - 1  # taken before prec follows the stream length (:973, :980-981)
+    w_pos = weight.clamp(0, 100)
+    w_neg = -(weight.clamp(-100, 0))
+    activation = activation.to(w_pos.dtype)
+    if forward == "full_or":
+        result_pos_value = linear_or_approx(activation, w_pos)
+        result_neg_value = linear_or_approx(activation, w_neg)
+    else:
+        result_pos_value = F.linear(activation, w_pos)
+        result_neg_value = F.linear(activation, w_neg)
+    if os.environ.get("Global_Sync", "1") == "1":
+        with torch.no_grad():
+            pos, neg = _ops.sc_linear_legacy(activation.data, weight.data, bit_length, 0 if forward == "full_or" else 51200,
+                                             weight_clamp=bit_range)
+            mean = lambda t: (t.to(torch.float32) / bit_length).to(torch.float16).to(result_pos_value.dtype)
+            result_pos_value.data = mean(pos)
+            result_neg_value.data = mean(neg)
+    return result_pos_value - result_neg_value

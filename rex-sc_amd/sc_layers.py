@@ -64,10 +64,18 @@ class Conv2d_Add_Partial(nn.Conv2d):
 
 
 class Linear_Or(nn.Linear):
-    """SC linear layer on the extension kernels (OR-n accumulation over the input features)."""
+    """SC linear layer (OR accumulation over the input features).
+
+    Default: the extension kernels' semantics (sc_matmul.cpp:576-676) with the keyword arguments of
+    Conv2d_Add_Partial (forward 'or_2', generator 'lfsr', err 6, load_unit, load_wait_w, sync, prec 7).
+    legacy=True: the reference's own Linear_Or (utils_class.py:183-208), which runs the legacy simulation
+    `linear_generic` (seeds 67/37/0, full OR accumulation): forward(input, prec=7, err=7, generator='lfsr')
+    quantises the input in place and the weight through QuantizeGrad, then calls
+    linear_generic(input, weight, bit_length=2**err, forward='full_or', generator=generator)."""
 
     def __init__(self, *kargs, **kwargs):
         self.run_args = {}
+        self.legacy = bool(kwargs.pop("legacy", False))
         for key, default in (("forward", "or_2"), ("generator", "lfsr"), ("err", 6), ("load_unit", 8),
                              ("load_wait_w", 1), ("sync", 1), ("prec", 7)):
             utils_f.setdict_default(self.run_args, kwargs, key, default)
@@ -75,7 +83,11 @@ class Linear_Or(nn.Linear):
         super(Linear_Or, self).__init__(*kargs, **kwargs)
         self.register_buffer("weight_flag", self.weight.data.clone())
 
-    def forward(self, input):
+    def forward(self, input, prec=7, err=7, generator="lfsr"):
+        if self.legacy:
+            input.data = utils_f.quantize(input.data, prec=prec)
+            weight = utils_f.QuantizeGrad.apply(self.weight, prec)
+            return utils_f.linear_generic(input, weight, bit_length=2 ** err, forward="full_or", generator=generator)
         input = utils_f.QuantizeGrad.apply(input, self.run_args["prec"])
         weight = utils_f.QuantizeGrad.apply(self.weight, self.run_args["prec"])
         keys = ("bit_length", "forward", "generator", "load_unit", "load_wait_w", "sync")

@@ -98,3 +98,18 @@ def check_calib_against_reference(fit):
 
 def test_calibration_fit_matches_reference_python():
     check_calib_against_reference(orc.compute_bias_std_coef)
+
+
+def _legacy_linear_cases():
+    g = np.load(os.path.join(ROOT, "tests", "golden", "ref_linear_legacy.npz"), allow_pickle=False)
+    return g, json.loads(bytes(g["meta"]).decode())
+
+
+@pytest.mark.parametrize("case", _legacy_linear_cases()[1], ids=lambda c: c["name"])
+def test_legacy_linear_generic_matches_reference_python(case):
+    """oracle.linear_generic_legacy against the vectors written by the reference's own linear_generic."""
+    g, _ = _legacy_linear_cases()
+    n = case["name"]
+    got = orc.linear_generic_legacy(g[n + "/x"], g[n + "/w"], case["bit_length"], case["forward"])
+    assert np.abs(g[n + "/y"]).max() > 0
+    assert np.array_equal(got, g[n + "/y"])
