@@ -30,7 +30,11 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "rex-sc_amd"))
 
-VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9  # lane-ops/s: 256 CUs x 4 SIMD16 x 2.4 GHz
+# Integer VALU roofs (lane-ops/s) at 256 CUs x 4 SIMDs x 2.4 GHz.  Measured per wave64 instruction and SIMD on this
+# part (profiles/valu_instruction_rates_gfx950.md): v_and_b32 2 cycles, v_bcnt_u32_b32 / v_and_or_b32 / v_pk_*_u16 4
+# cycles.  The and + popcount pair therefore retires in 6 cycles: 2 x 64 lane-ops / 6 cycles per SIMD.
+VALU_PEAK_4CYCLE = 256 * 4 * 16 * 2.4e9          # every instruction at 4 cycles: 39.32 T lane-op/s
+VALU_PEAK_LANEOPS = 256 * 4 * (2 * 64 / 6) * 2.4e9  # the and + popcount pair: 52.43 T lane-op/s
 HBM_PEAK = 8.0e12
 
 # (C_in, H_in, C_out, K, stride) for the 19 SC convs of ResNet-18 at 224x224 input
@@ -88,6 +92,7 @@ def main():
 
     import torch
     import _lib
+    import _ops
     import sc_extension_cuda
 
     if not torch.cuda.is_available():
@@ -142,14 +147,20 @@ def main():
     achieved = dom["total_work"] / (dom["total_ms"] * 1e-3)
     comp_ms = sum(v["total_ms"] for v in comp.values())
     comp_ops = sum(v["total_work"] for v in comp.values())
+    # what the register-only and/popcount probe kernel sustains on this machine, beside the nominal peak
+    peak_measured = max(_lib.valu_probe(0, 2000) for _ in range(2))
+    traffic = quoted_traffic()
     roofline = {
         "bound": "valu", "kernel": dom_name,
         "achieved": achieved / 1e12, "peak": VALU_PEAK_LANEOPS / 1e12, "unit": "Tlane-op/s",
         "frac": achieved / VALU_PEAK_LANEOPS,
-        # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the stage-2
-        # 3x3 layer (profiles/sc_compute_3x3_c128_hbm_traffic.md): 39.5 MB read + 25.7 MB written
-        # against 56.4 MB algorithmic; at these rates the kernel is nowhere near the HBM roof.
-        "traffic": 65.2e6, "traffic_shape": "128->128 3x3 28x28 batch 64",
+        "peak_model": "and+popcount pair at its measured instruction costs (v_and_b32 2 cycles + v_bcnt_u32_b32 4 cycles per "
+                      "wave64 and SIMD); every instruction at 4 cycles would be %.2f" % (VALU_PEAK_4CYCLE / 1e12),
+        "peak_measured": peak_measured / 1e12, "frac_of_peak_measured": achieved / peak_measured,
+        "peak_measured_and_or": _lib.valu_probe(1, 2000) / 1e12,
+        # HBM bytes per launch of this kernel: quoted from the committed rocprofv3 counter summary (FETCH_SIZE +
+        # WRITE_SIZE on one layer shape), not measured in this run; null when the summary is absent
+        "traffic": traffic.get("bytes"), "traffic_shape": traffic.get("shape"), "traffic_source": traffic.get("source"),
         "avg_launch_us": dom["total_ms"] * 1e3 / dom["calls"], "launches": dom["calls"],
         "all_compute_kernels_frac": comp_ops / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS,
         "whole_step_frac": (total_mac * L * 4 / 32) / sec / VALU_PEAK_LANEOPS,
@@ -164,20 +175,45 @@ def main():
         "config": {"workload": ("resnet18_sc_conv_forward: 19 SC conv layers (16 3x3 + 3 1x1), batch %d, OR-%d, "
                                 "%d-bit streams, channels_last, float in / int16 pos+neg out" % (N, OR_N, L))
                                if not args.only_layer else "single SC conv layer C,H,O,K,S=%s, batch %d" % (args.only_layer, N),
-                   "batch": N, "bit_length": L, "or_n": OR_N, "images_per_s": N / sec},
+                   "batch": N, "bit_length": L, "or_n": OR_N, "images_per_s": N / sec,
+                   "xnor_mode": _ops.xnor_mode()},
         "roofline": roofline,
     }
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, L, OR_N)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, L, OR_N, full_batch=N)
     if not args.no_extra:
         try:
             import bench_extra
             out["extra"] = bench_extra.run(torch, dev)
+            if not args.no_cpu_baseline:
+                for name, base in cpu_baselines_other_configs(torch).items():
+                    target = out["extra"].get(name.split("/")[0], {})
+                    if "/" in name:
+                        target = target.get("shapes", {}).get(name.split("/")[1], {})
+                    if isinstance(target, dict) and "error" not in target:
+                        target["cpu_baseline"] = base
         except Exception as e:  # the headline must survive a failure of an auxiliary config
             out["extra"] = {"error": "%s: %s" % (type(e).__name__, e)}
     print(json.dumps(out))
     return 0
+
+
+def quoted_traffic():
+    """HBM bytes per launch of the dominant compute kernel as the committed counter summary states them (a line
+    `traffic_bytes_per_launch: <number>` and a line `traffic_shape: <text>`)."""
+    import re
+    path = os.path.join(ROOT, "profiles", "sc_compute_3x3_c128_hbm_traffic.md")
+    try:
+        text = open(path).read()
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
+        sh = re.search(r"^traffic_shape:\s*(.+)$", text, re.M)
+        if m:
+            return {"bytes": float(m.group(1)), "shape": sh.group(1).strip() if sh else None,
+                    "source": "profiles/" + os.path.basename(path)}
+    except OSError:
+        pass
+    return {}
 
 
 _REF_CHILD = r"""
@@ -186,11 +222,12 @@ sys.path.insert(0, sys.argv[1])
 import numpy as np, torch
 import sc_extension
 layers = json.loads(sys.argv[2]); batch = int(sys.argv[3]); L = int(sys.argv[4]); or_n = int(sys.argv[5])
-rng = np.random.default_rng(5)
+full = int(sys.argv[6])
 ops = []
-for (C, H, O, K, s) in layers:
-    x = torch.from_numpy((rng.integers(0, L, size=(batch, C, H, H)) / L).astype(np.float32))
-    w = torch.from_numpy((rng.integers(-L + 1, L, size=(O, C, K, K)) / L).astype(np.float32))
+for i, (C, H, O, K, s) in enumerate(layers):
+    g = torch.Generator().manual_seed(500 + i)   # the tensors of the GPU leg, first `batch` images
+    x = (torch.randint(0, L, (full, C, H, H), generator=g).float() / L)[:batch]
+    w = torch.randint(-L + 1, L, (O, C, K, K), generator=g).float() / L
     ops.append((x.contiguous(memory_format=torch.channels_last), w, K, s))
 t0 = time.perf_counter()
 for (x, w, K, s) in ops:
@@ -199,7 +236,7 @@ print(json.dumps({"sec": time.perf_counter() - t0, "threads": torch.get_num_thre
 """
 
 
-def cpu_baseline(sample_batch, L, or_n):
+def cpu_baseline(sample_batch, L, or_n, full_batch=64):
     """CPU rate of the same 19 layers on this host, on a bounded sample (bit-MAC/s scales linearly
     with batch for this embarrassingly parallel op).  Preferred: the reference's own CPU extension,
     compiled from its sources into oracle/_ref/ (kind "reference"), run in a child process so that a
@@ -209,19 +246,22 @@ def cpu_baseline(sample_batch, L, or_n):
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import numpy as np
     import oracle as orc
+    import torch
     cores = orc.num_threads()
-    rng = np.random.default_rng(5)
+    sample_batch = min(sample_batch, full_batch)
     mac = 0
-    t0 = time.perf_counter()
-    for (C, H, O, K, s) in RESNET18_SC_LAYERS:
-        x = (rng.integers(0, L, size=(sample_batch, C, H, H)) / L).astype(np.float32)
-        w = (rng.integers(-L + 1, L, size=(O, C, K, K)) / L).astype(np.float32)
+    sec = 0.0
+    for i, (C, H, O, K, s) in enumerate(RESNET18_SC_LAYERS):
+        # the same tensors as the GPU leg (same seeds, same generator calls), first sample_batch images
+        xt, wt = make_conv_operands(torch, full_batch, C, H, O, K, L, seed=500 + i)
+        x, w = xt[:sample_batch].numpy(), wt.numpy()
+        t0 = time.perf_counter()
         orc.conv2d_generic_general_split(x, w, L, -1, 16, (K // 2, K // 2), (s, s), (7, 8, 1), or_n - 1, 1,
                                          channels_last_activation=True)
+        sec += time.perf_counter() - t0
         mac += layer_macs(sample_batch, C, H, O, K, s)
-    sec = time.perf_counter() - t0
     port = {"value": mac * L / sec, "unit": "bit-MAC/s", "cores": cores, "kind": "port",
-            "sample": "same 19 ResNet-18 SC conv layers at batch %d (%.1f s of CPU time on %d threads)"
+            "sample": "the GPU leg's tensors, same 19 ResNet-18 SC conv layers, first %d images (%.1f s of CPU time on %d threads)"
                       % (sample_batch, sec, cores)}
     ref_dir = os.path.join(ROOT, "oracle", "_ref")
     ref_batch = max(1, sample_batch // 4)
@@ -230,16 +270,53 @@ def cpu_baseline(sample_batch, L, or_n):
         return port
     try:
         out = subprocess.run([sys.executable, "-c", _REF_CHILD, ref_dir, json.dumps(RESNET18_SC_LAYERS), str(ref_batch),
-                              str(L), str(or_n)], capture_output=True, text=True, timeout=180)
+                              str(L), str(or_n), str(full_batch)], capture_output=True, text=True, timeout=180)
         res = json.loads(out.stdout.strip().splitlines()[-1])
         rmac = sum(layer_macs(ref_batch, C, H, O, K, s) for (C, H, O, K, s) in RESNET18_SC_LAYERS)
         return {"value": rmac * L / res["sec"], "unit": "bit-MAC/s", "cores": res["threads"], "kind": "reference",
-                "sample": "same 19 ResNet-18 SC conv layers at batch %d through the reference's compiled CPU extension "
-                          "(%.1f s on %d threads)" % (ref_batch, res["sec"], res["threads"]),
+                "sample": "the GPU leg's tensors, same 19 ResNet-18 SC conv layers, first %d images, through the reference's "
+                          "compiled CPU extension (%.1f s on %d threads)" % (ref_batch, res["sec"], res["threads"]),
                 "port_value": port["value"], "port_sample": port["sample"]}
     except Exception as e:  # missing build, illegal instruction, timeout: report the port
         port["reference_skipped"] = "%s: %s" % (type(e).__name__, str(e)[:200])
         return port
+
+
+def cpu_baselines_other_configs(torch):
+    """The C restatement in oracle/ (kind "port", OpenMP) on the tensors bench_extra.py builds for configurations 1, 2
+    and 4 (same seeds, same generator calls): configurations 1 and 2 at full size, the fixed-point conv on the first two
+    images of each shape."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as orc
+    cores = orc.num_threads()
+    res = {}
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randint(0, 32, (32, 32, 32, 32), generator=g).float() / 32).numpy()
+    w = ((torch.rand(64, 32, 3, 3, generator=g) * 2 - 1) * 32).round().clamp(-31, 31).div(32).numpy()
+    t0 = time.perf_counter()
+    orc.conv2d_generic_general_split(x, w, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 0, 1)
+    sec = time.perf_counter() - t0
+    res["config1_sc_conv_or1"] = {"value": 32 * 32 * 32 * 64 * 32 * 9 * 32 / sec, "unit": "bit-MAC/s", "cores": cores,
+                                  "kind": "port", "sample": "the same tensors at full size (%.2f s)" % sec}
+    g = torch.Generator().manual_seed(2)
+    x = (torch.randint(0, 64, (256, 4096), generator=g).float() / 64).numpy()
+    w = ((torch.rand(1024, 4096, generator=g) * 2 - 1) * 64).round().clamp(-63, 63).div(64).numpy()
+    t0 = time.perf_counter()
+    orc.linear_generic_general(x, w, (7, 8, 1), 64, -1, 1, 1)
+    sec = time.perf_counter() - t0
+    res["config2_sc_linear"] = {"value": 256 * 4096 * 1024 * 64 / sec, "unit": "bit-MAC/s", "cores": cores, "kind": "port",
+                                "sample": "the same tensors at full size (%.2f s)" % sec}
+    for C, H in ((64, 56), (128, 28), (256, 14), (512, 7)):
+        g = torch.Generator().manual_seed(4)
+        x = (torch.randint(0, 32, (64, C, H, H), generator=g).float() / 32)[:2].numpy()
+        w = (torch.randint(-31, 32, (C, C, 3, 3), generator=g).float() / 32).numpy()
+        t0 = time.perf_counter()
+        orc.conv2d_saturate(x, w, 0, 5, 24, (1, 1), (1, 1))
+        sec = time.perf_counter() - t0
+        res["config4_fixed_conv/%dx%dx%d" % (C, H, H)] = {
+            "value": 2 / sec, "unit": "images/s", "cores": cores, "kind": "port",
+            "sample": "the first 2 images of the same tensors (%.2f s)" % sec}
+    return res
 
 
 if __name__ == "__main__":

@@ -1,17 +1,30 @@
 """The other reference configurations, reported next to the headline of bench.py.
 
-Each entry states its workload, the time of one pass, a rate in the unit that fits it and, where
-one kernel dominates, the fraction of the roofline that bounds it (VALU integer throughput for the
-AND/popcount kernels, HBM bandwidth for the streaming kernels).  Everything runs on one GPU with
-synthetic data; the train steps follow the reference's step structure (utils_own.py:96-171):
-forward, label-smoothed cross entropy, backward, Adam step, in the three flavours the training
-loop alternates between (sync 1 = SC forward, 3 = error injection only, 2 = calibration on half
-a batch).
+Each entry states its workload, the time of one pass, a rate in the unit that fits it and the fraction
+of the roofline that bounds its kernels (VALU integer throughput for the AND/popcount kernels, HBM
+bandwidth for the streaming kernels).  Everything runs on one GPU with synthetic data; the train steps
+follow the reference's step structure (utils_own.py:96-171): forward, label-smoothed cross entropy,
+backward, Adam step, in the three flavours the training loop alternates between (sync 1 = SC forward,
+3 = error injection only, 2 = calibration on half a batch).
+
+Kernel-level figures come from the library's own HIP-event brackets (rexsc_profile_begin / _end) in a
+pass separate from the wall-clock timing.  The streaming kernels are timed twice: on one set of buffers
+(which the 256 MB memory-side cache can partly hold) and rotating through more than 1 GiB of distinct
+buffers, so that every byte comes from and goes to HBM; `hbm_frac` is the rotating figure.
 """
+import ctypes
 import time
 
-VALU_PEAK_LANEOPS = 256 * 64 * 2.4e9
+# integer VALU roofs, lane-ops/s (see bench.py): and + popcount pair at 2 + 4 cycles per wave64 and SIMD; single
+# instructions of the 4-cycle class (v_and_or_b32, the OR-1 kernels)
+VALU_PEAK_LANEOPS = 256 * 4 * (2 * 64 / 6) * 2.4e9
+VALU_PEAK_4CYCLE = 256 * 4 * 16 * 2.4e9
 HBM_PEAK = 8.0e12
+ROTATE_BYTES = 1.25 * 2 ** 30  # distinct bytes touched before a buffer is used again
+
+SC_KERNELS = ("sc_compute", "sc_finalize", "sng_")
+STREAM_KERNELS = ("orn_", "sc_counts_to_float", "quantize", "split_weight", "merge_weight_grad", "calib_stats",
+                  "fixed_")
 
 
 def _time(torch, fn, steps, warmup):
@@ -25,47 +38,102 @@ def _time(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def _profile(torch, fn, reps):
+    """Per-kernel records of `reps` passes of fn: {name: dict(calls, total_ms, total_work)} per pass."""
+    import _lib
+    fn()
+    torch.cuda.synchronize()
+    _lib.profile_begin()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    prof = _lib.profile_end(max_records=128)
+    return {k: dict(calls=v["calls"] / reps, ms=v["total_ms"] / reps, work=v["total_work"] / reps) for k, v in prof.items()}
+
+
+def _breakdown(prof, step_ms):
+    """Library time of one step by kernel class, with the roofline fraction of each class."""
+    sc = {k: v for k, v in prof.items() if k.startswith(SC_KERNELS)}
+    comp = {k: v for k, v in sc.items() if k.startswith("sc_compute")}
+    pw = {k: v for k, v in prof.items() if k.startswith(STREAM_KERNELS)}
+    sc_ms = sum(v["ms"] for v in sc.values())
+    comp_ms = sum(v["ms"] for v in comp.values())
+    comp_ops = sum(v["work"] for v in comp.values())
+    pw_ms = sum(v["ms"] for v in pw.values())
+    pw_bytes = sum(v["work"] for v in pw.values())
+    lib_ms = sc_ms + pw_ms
+    out = {
+        "sc_kernels_ms": round(sc_ms, 4), "sc_compute_ms": round(comp_ms, 4),
+        "sc_compute_valu_frac": comp_ops / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS if comp_ms else None,
+        "sc_kernels_valu_frac": comp_ops / (sc_ms * 1e-3) / VALU_PEAK_LANEOPS if sc_ms else None,
+        "streaming_kernels_ms": round(pw_ms, 4),
+        "streaming_kernels_hbm_frac": pw_bytes / (pw_ms * 1e-3) / HBM_PEAK if pw_ms else None,
+        "library_ms": round(lib_ms, 4),
+        # kernels of this library against the step's wall clock; at sync 1 the SC forward runs on a second stream
+        # beside the float convolution, so the two shares can add up to more than one
+        "share_outside_library": max(0.0, 1.0 - lib_ms / step_ms),
+        "kernel_ms": {k: round(v["ms"], 4) for k, v in sorted(prof.items())},
+    }
+    return out
+
+
 def config1_sc_conv_or1(torch, dev):
     import sc_extension_cuda
     L = 32
     g = torch.Generator().manual_seed(1)
-    x = (torch.randint(0, 32, (32, 32, 32, 32), generator=g).float() / 32).to(dev)
-    w = ((torch.rand(64, 32, 3, 3, generator=g) * 2 - 1) * 32).round().clamp(-31, 31).div(32).to(dev)
+    xc = torch.randint(0, 32, (32, 32, 32, 32), generator=g).float() / 32
+    wc = ((torch.rand(64, 32, 3, 3, generator=g) * 2 - 1) * 32).round().clamp(-31, 31).div(32)
+    x, w = xc.to(dev), wc.to(dev)
     fn = lambda: sc_extension_cuda.conv2d_generic_general_split_acc(x, w, L, -1, 16, (1, 1), (1, 1), (7, 8, 1), 0, 1,
                                                                     True, False)
     sec = _time(torch, fn, 50, 5)
+    prof = _profile(torch, fn, 5)
     mac = 32 * 32 * 32 * 64 * 32 * 9
-    return {"workload": "SC conv2d forward OR-1, 32-bit streams, N32 C32 32x32 -> 64, 3x3 s1 p1, NCHW",
-            "ms": sec * 1e3, "bit_mac_per_s": mac * L / sec, "images_per_s": 32 / sec,
-            "valu_frac": mac * L * 4 / 32 / sec / VALU_PEAK_LANEOPS}
+    words = mac * L / 32  # 32-channel stream words ANDed per polarity
+    comp_ms = sum(v["ms"] for k, v in prof.items() if k.startswith("sc_compute"))
+    out = {"workload": "SC conv2d forward OR-1, 32-bit streams, N32 C32 32x32 -> 64, 3x3 s1 p1, NCHW",
+           "ms": sec * 1e3, "bit_mac_per_s": mac * L / sec, "images_per_s": 32 / sec,
+           # op model: the AND/popcount formulation costs 2 VALU ops per word and polarity; saturation at one needs no
+           # count, and this kernel issues ONE v_and_or_b32 per word and polarity -- both fractions are stated
+           "op_model": "kernel issues 1 op/word/polarity (v_and_or_b32); the 2-op figure prices the and+popcount formulation",
+           # 2-op model against the pair roof (52.43 T); 1-op model against the roof of the instruction issued (39.32 T)
+           "valu_frac_2op": words * 4 / sec / VALU_PEAK_LANEOPS, "valu_frac_1op": words * 2 / sec / VALU_PEAK_4CYCLE,
+           "sc_compute_ms": comp_ms,
+           "sc_compute_valu_frac_1op": words * 2 / (comp_ms * 1e-3) / VALU_PEAK_4CYCLE if comp_ms else None,
+           "kernel_ms": {k: round(v["ms"], 4) for k, v in sorted(prof.items())}}
+    return out
 
 
 def config2_sc_linear(torch, dev):
+    import sc_extension_cuda
     import sc_functional as uf
     L = 64
     g = torch.Generator().manual_seed(2)
-    x = (torch.randint(0, 64, (256, 4096), generator=g).float() / 64).to(dev).requires_grad_(True)
-    w = ((torch.rand(1024, 4096, generator=g) * 2 - 1) * 64).round().clamp(-63, 63).div(64).to(dev).requires_grad_(True)
+    xc = torch.randint(0, 64, (256, 4096), generator=g).float() / 64
+    wc = ((torch.rand(1024, 4096, generator=g) * 2 - 1) * 64).round().clamp(-63, 63).div(64)
+    x = xc.to(dev).requires_grad_(True)
+    w = wc.to(dev).requires_grad_(True)
     gout = torch.randn(256, 1024, generator=g).to(dev)
-
-    def fwd():
-        return uf.linear_generic_sc(x, w, bit_length=L, forward="or_2", generator="lfsr", sync=1)
 
     def fwd_bwd():
         x.grad = None
         w.grad = None
-        fwd().backward(gout)
+        uf.linear_generic_sc(x, w, bit_length=L, forward="or_2", generator="lfsr", sync=1).backward(gout)
 
     with torch.no_grad():
-        import sc_extension_cuda
         sc_only = lambda: sc_extension_cuda.linear_generic_general_acc(x, w, (7, 8, 1), L, -1, 1, 1, True, False)
         sec_sc = _time(torch, sc_only, 20, 3)
+        prof = _profile(torch, sc_only, 5)
     sec_fb = _time(torch, fwd_bwd, 20, 3)
     mac = 256 * 4096 * 1024
-    return {"workload": "SC linear OR-2, 64-bit streams, 256x4096 . (1024x4096)^T; backward through the float surrogate",
-            "sc_forward_ms": sec_sc * 1e3, "forward_backward_ms": sec_fb * 1e3,
-            "bit_mac_per_s": mac * L / sec_sc, "samples_per_s_fwd_bwd": 256 / sec_fb,
-            "valu_frac": mac * L * 4 / 32 / sec_sc / VALU_PEAK_LANEOPS}
+    comp_ms = sum(v["ms"] for k, v in prof.items() if k.startswith("sc_compute"))
+    out = {"workload": "SC linear OR-2, 64-bit streams, 256x4096 . (1024x4096)^T; backward through the float surrogate",
+           "sc_forward_ms": sec_sc * 1e3, "forward_backward_ms": sec_fb * 1e3,
+           "bit_mac_per_s": mac * L / sec_sc, "samples_per_s_fwd_bwd": 256 / sec_fb,
+           "valu_frac": mac * L * 4 / 32 / sec_sc / VALU_PEAK_LANEOPS,
+           "sc_compute_valu_frac": mac * L * 4 / 32 / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS if comp_ms else None,
+           "kernel_ms": {k: round(v["ms"], 4) for k, v in sorted(prof.items())}}
+    return out
 
 
 def _train_flavours(torch, dev, net, make_batch, batch, steps, lr):
@@ -87,6 +155,7 @@ def _train_flavours(torch, dev, net, make_batch, batch, steps, lr):
 
         sec = _time(torch, step, steps, 2)
         out[name] = {"ms_per_step": sec * 1e3, "images_per_s": n / sec, "batch": n}
+        out[name].update(_breakdown(_profile(torch, step, 2), sec * 1e3))
     return out
 
 
@@ -106,17 +175,45 @@ def config3_tinyconv_step(torch, dev):
     return res
 
 
+def _rotating_sets(nbytes_per_set):
+    return max(2, int(ROTATE_BYTES // max(1, nbytes_per_set)) + 1)
+
+
 def config4_fixed_conv(torch, dev):
+    import _lib
     import fixed_extension_cuda
     import sc_functional as uf
+    L_ = _lib.lib()
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ptr = lambda t: ctypes.c_void_p(t.data_ptr())
     out = {"workload": "saturating fixed-point conv (add_config 0, 5-bit operands, 24-bit accumulator), batch 64, "
-                       "conv3x3 s1 p1: forward kernel alone, and forward + backward through the float conv", "shapes": {}}
+                       "conv3x3 s1 p1: forward op alone (one buffer set, and rotating through >1 GiB of distinct "
+                       "buffers), and forward + backward through the float conv", "shapes": {}}
     for C, H in ((64, 56), (128, 28), (256, 14), (512, 7)):
         g = torch.Generator().manual_seed(4)
-        x = (torch.randint(0, 32, (64, C, H, H), generator=g).float() / 32).to(dev)
-        w = (torch.randint(-31, 32, (C, C, 3, 3), generator=g).float() / 32).to(dev)
+        xc = torch.randint(0, 32, (64, C, H, H), generator=g).float() / 32
+        wc = torch.randint(-31, 32, (C, C, 3, 3), generator=g).float() / 32
+        x, w = xc.to(dev), wc.to(dev)
         fn = lambda: fixed_extension_cuda.conv2d_saturate_acc(x, w, 0, 5, 24, (1, 1), (1, 1))
         sec = _time(torch, fn, 10, 2)
+        nbytes = 4 * x.numel() + 4 * w.numel() + 4 * 64 * C * H * H
+        # rotating: distinct input / weight / output / workspace per call, through the C ABI
+        d = _lib.FixedDesc(64, C, H, H, C, 3, 3, 1, 1, 1, 1, 0, 5, 24)
+        ws_bytes = L_.rexsc_fixed_conv2d_workspace_bytes(ctypes.byref(d))
+        nset = _rotating_sets(nbytes)
+        sets = [(x.clone(), w.clone(), torch.empty((64, C, H, H), dtype=torch.int32, device=dev)) for _ in range(nset)]
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+        state = {"i": 0}
+
+        def rot():
+            xs, wsx, os_ = sets[state["i"] % nset]
+            state["i"] += 1
+            _lib.check(L_.rexsc_fixed_conv2d(ctypes.byref(d), ptr(xs), ptr(wsx), ptr(os_), ptr(ws), ws.numel(), stream()),
+                       "rexsc_fixed_conv2d")
+
+        sec_rot = _time(torch, rot, 2 * nset, nset)
+        prof = _profile(torch, rot, nset)
+        del sets
         # forward + backward as the training path runs it: fixed-point forward values over the float
         # conv, whose backward supplies the gradients (generator 'fixed', forward 'full_bin')
         xg, wg = x.clone().requires_grad_(True), w.clone().requires_grad_(True)
@@ -129,12 +226,18 @@ def config4_fixed_conv(torch, dev):
                               sync=1).backward(gout)
 
         sec_fb = _time(torch, fwd_bwd, 10, 3)
-        nbytes = 4 * x.numel() + 4 * w.numel() + 4 * 64 * C * H * H
         mac = 64 * H * H * C * C * 9
-        out["shapes"]["%dx%dx%d" % (C, H, H)] = {"ms": sec * 1e3, "GB_per_s": nbytes / sec / 1e9,
-                                               "hbm_frac": nbytes / sec / HBM_PEAK, "mac_per_s": mac / sec,
-                                               "images_per_s": 64 / sec, "forward_backward_ms": sec_fb * 1e3,
-                                               "images_per_s_fwd_bwd": 64 / sec_fb}
+        kern_ms = sum(v["ms"] for v in prof.values())
+        entry = {"ms": sec * 1e3, "ms_rotating": sec_rot * 1e3, "rotating_sets": nset,
+                 "kernel_ms_rotating": {k: round(v["ms"], 4) for k, v in sorted(prof.items())},
+                 "GB_per_s": nbytes / sec_rot / 1e9, "hbm_frac": nbytes / sec_rot / HBM_PEAK,
+                 "hbm_frac_kernels_only": nbytes / (kern_ms * 1e-3) / HBM_PEAK if kern_ms else None,
+                 "hbm_frac_one_buffer_set": nbytes / sec / HBM_PEAK,
+                 "mac_per_s": mac / sec_rot, "images_per_s": 64 / sec_rot, "forward_backward_ms": sec_fb * 1e3,
+                 "images_per_s_fwd_bwd": 64 / sec_fb}
+        out["shapes"]["%dx%dx%d" % (C, H, H)] = entry
+        del x, w, xg, wg
+        torch.cuda.empty_cache()
     return out
 
 
@@ -151,6 +254,13 @@ def config5_resnet18_step(torch, dev, batch=64):
     res = _train_flavours(torch, dev, net, make_batch, batch, 5, 1e-3)
     res["workload"] = ("ResNet-18 SC training step, batch %d, 3x224x224, channels_last, OR-2, 32-bit streams, "
                        "float stem/fc, Adam" % batch)
+    # evaluation: weights frozen, the layers reuse their weight streams from call to call
+    net.eval()
+    net.sync = 1
+    x, _ = make_batch(batch)
+    with torch.no_grad():
+        sec = _time(torch, lambda: net(x), 5, 2)
+    res["eval_forward_no_grad"] = {"ms": sec * 1e3, "images_per_s": batch / sec}
     return res
 
 
@@ -176,40 +286,75 @@ def resnet18_sc_conv_fwd_bwd(torch, dev, batch=64):
                               sync=1).backward(gout)
 
     sec = _time(torch, step, 5, 2)
-    return {"workload": "19 ResNet-18 SC conv layers, batch %d, OR-2, 32-bit streams, channels_last: SC forward + "
-                        "backward through the float surrogate (conv2d_generic, sync 1)" % batch,
-            "ms_per_step": sec * 1e3, "images_per_s": batch / sec}
+    res = {"workload": "19 ResNet-18 SC conv layers, batch %d, OR-2, 32-bit streams, channels_last: SC forward + "
+                       "backward through the float surrogate (conv2d_generic, sync 1)" % batch,
+           "ms_per_step": sec * 1e3, "images_per_s": batch / sec}
+    res.update(_breakdown(_profile(torch, step, 2), sec * 1e3))
+    return res
 
 
 def pointwise(torch, dev):
-    import _ops
-    n = 64 * 64 * 56 * 56  # one ResNet-18 layer1 activation tensor
-    x = torch.rand(n, device=dev) * 4
-    x2 = torch.rand(n, device=dev) * 4
-    gout = torch.randn(n, device=dev)
-    coef = torch.tensor([0.01, -0.01, 0.002, 0.0, 0.0, 0.0], device=dev)
-    res = {"workload": "pointwise kernels on %d float32 elements (64x64x56x56)" % n}
-    for name, fn, bpe in (
-            ("orn_forward", lambda: _ops.orn_forward(x, 2), 8),
-            ("orn_backward", lambda: _ops.orn_backward(gout, x, 2), 12),
-            ("orn_bias_std_both_forward", lambda: _ops.orn_bias_std_both_forward(x, x2, coef, coef, 2), 12),
-            ("orn_bias_std_both_backward", lambda: _ops.orn_bias_std_both_backward(gout, x, x2, coef, 2), 20)):
-        sec = _time(torch, fn, 20, 3)
-        res[name] = {"ms": sec * 1e3, "GB_per_s": bpe * n / sec / 1e9, "hbm_frac": bpe * n / sec / HBM_PEAK}
-    # the kernels of the merged surrogate: both polarities in one [pixels][2][channels] tensor
+    """The streaming kernels on one ResNet-18 layer1 activation tensor, through the C ABI with preallocated
+    outputs: on one buffer set, and rotating through more than 1 GiB of distinct inputs and outputs."""
+    import _lib
+    L_ = _lib.lib()
+    n = 64 * 64 * 56 * 56
     outer, inner = 64 * 56 * 56, 64
-    s2 = (torch.rand(64, 2 * inner, 56, 56, device=dev) * 4).contiguous(memory_format=torch.channels_last)
-    g4 = gout.view(64, 56, 56, inner).permute(0, 3, 1, 2)
-    pos = torch.randint(0, 64, (64, inner, 56, 56), device=dev, dtype=torch.int16).contiguous(memory_format=torch.channels_last)
-    neg = torch.randint(0, 64, (64, inner, 56, 56), device=dev, dtype=torch.int16).contiguous(memory_format=torch.channels_last)
-    for name, fn, bpe in (
-            ("orn_pair_backward", lambda: _ops.orn_pair_backward(g4, s2, outer, inner, True, 2), 20),
-            ("orn_bias_std_pair_forward", lambda: _ops.orn_bias_std_pair_forward(s2, outer, inner, True, coef, coef, 2), 12),
-            ("orn_bias_std_pair_backward", lambda: _ops.orn_bias_std_pair_backward(g4, s2, outer, inner, True, coef, 2), 20),
-            ("sc_counts_to_float", lambda: _ops.sc_counts_to_float(pos, neg, 32), 8),
-            ("quantize", lambda: _ops.quantize(x, 7), 8)):
-        sec = _time(torch, fn, 20, 3)
-        res[name] = {"ms": sec * 1e3, "GB_per_s": bpe * n / sec / 1e9, "hbm_frac": bpe * n / sec / HBM_PEAK}
+    coef = torch.tensor([0.01, -0.01, 0.002, 0.0, 0.0, 0.0], device=dev)
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    f32 = lambda k: torch.rand(k, device=dev) * 4
+    i16 = lambda k: torch.randint(0, 64, (k,), device=dev, dtype=torch.int16)
+    e32 = lambda k: torch.empty(k, dtype=torch.float32, device=dev)
+    # name -> (bytes per element of y, buffer makers, call)
+    kernels = {
+        "orn_forward": (8, lambda: (f32(n), e32(n)),
+                        lambda b: L_.rexsc_orn_forward(p(b[0]), p(b[1]), n, 2, stream())),
+        "orn_backward": (12, lambda: (f32(n), f32(n), e32(n)),
+                         lambda b: L_.rexsc_orn_backward(p(b[0]), p(b[1]), p(b[2]), n, 2, 1, stream())),
+        "orn_bias_std_both_forward": (12, lambda: (f32(n), f32(n), e32(n)),
+                                      lambda b: L_.rexsc_orn_bias_std_both_forward(p(b[0]), p(b[1]), p(coef), p(coef), p(b[2]), n, 2,
+                                                                                   1234, 0, None, None, None, stream())),
+        "orn_bias_std_both_backward": (20, lambda: (f32(n), f32(n), f32(n), e32(n), e32(n)),
+                                       lambda b: L_.rexsc_orn_bias_std_both_backward(p(b[0]), p(b[1]), p(b[2]), p(coef), p(b[3]),
+                                                                                     p(b[4]), n, 2, 1, stream())),
+        "orn_pair_backward": (20, lambda: (f32(n), f32(2 * n), e32(2 * n)),
+                              lambda b: L_.rexsc_orn_pair_backward(p(b[0]), p(b[1]), p(b[2]), outer, inner, 2, 1, stream())),
+        "orn_bias_std_pair_forward": (12, lambda: (f32(2 * n), e32(n)),
+                                      lambda b: L_.rexsc_orn_bias_std_pair_forward(p(b[0]), p(coef), p(coef), p(b[1]), outer, inner, 2,
+                                                                                   1234, 0, None, stream())),
+        "orn_bias_std_pair_backward": (20, lambda: (f32(n), f32(2 * n), e32(2 * n)),
+                                       lambda b: L_.rexsc_orn_bias_std_pair_backward(p(b[0]), p(b[1]), p(coef), p(b[2]), outer, inner,
+                                                                                     2, 1, stream())),
+        "sc_counts_to_float": (8, lambda: (i16(n), i16(n), e32(n)),
+                               lambda b: L_.rexsc_sc_counts_to_float(p(b[0]), p(b[1]), p(b[2]), n, 32, stream())),
+        "quantize": (8, lambda: (f32(n), e32(n)),
+                     lambda b: L_.rexsc_quantize(p(b[0]), p(b[1]), n, 7, stream())),
+    }
+    res = {"workload": "streaming kernels on %d float32 elements (64x64x56x56); hbm_frac: rotating through >1 GiB of "
+                       "distinct buffers; hbm_frac_one_buffer_set: the same buffers every call" % n}
+    for name, (bpe, make, call) in kernels.items():
+        one = make()
+        sec_one = _time(torch, lambda: _lib.check(call(one), name), 20, 3)
+        set_bytes = sum(t.numel() * t.element_size() for t in one)
+        nset = _rotating_sets(set_bytes)
+        sets = [one] + [make() for _ in range(nset - 1)]
+        state = {"i": 0}
+
+        def rot():
+            b = sets[state["i"] % nset]
+            state["i"] += 1
+            _lib.check(call(b), name)
+
+        sec = _time(torch, rot, 2 * nset, nset)
+        prof = _profile(torch, rot, nset)
+        kms = prof.get(name, {}).get("ms")
+        res[name] = {"ms": sec * 1e3, "kernel_ms": kms, "rotating_sets": nset, "GB_per_s": bpe * n / sec / 1e9,
+                     "hbm_frac": bpe * n / sec / HBM_PEAK,
+                     "hbm_frac_kernel_only": bpe * n / (kms * 1e-3) / HBM_PEAK if kms else None,
+                     "hbm_frac_one_buffer_set": bpe * n / sec_one / HBM_PEAK}
+        del sets, one
+        torch.cuda.empty_cache()
     return res
 
 

@@ -239,6 +239,12 @@ typedef struct rexsc_profile_record {
 int rexsc_profile_begin(void);
 int rexsc_profile_end(rexsc_profile_record *out, int max_records);
 
+/* Integer VALU peak probe (no counterpart in the reference): runs a register-only kernel that issues the SC
+ * compute kernel's instruction pair (mode 0: v_and_b32 + v_bcnt_u32_b32 accumulate; mode 1: v_and_or_b32)
+ * with eight waves per SIMD and returns its duration and the lane-operations it executed, so that roofline
+ * fractions can be quoted against a peak measured on the machine at hand.  Synchronises the stream. */
+int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream, double *ms_out, double *lane_ops_out);
+
 #ifdef __cplusplus
 }
 #endif

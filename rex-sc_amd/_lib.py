@@ -72,6 +72,7 @@ SIGNATURES = {
     "rexsc_fixed_conv2d": (_int, [ctypes.POINTER(FixedDesc), _vp, _vp, _vp, _vp, _sz, _vp]),
     "rexsc_profile_begin": (_int, []),
     "rexsc_profile_end": (_int, [ctypes.POINTER(ProfileRecord), _int]),
+    "rexsc_valu_probe": (_int, [_int, _int, _vp, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_double)]),
     "rexsc_calib_stats": (_int, [_vp, _vp, _sz, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float),
                                  _int, _vp, _vp]),
 }
@@ -110,3 +111,10 @@ def profile_end(max_records=64):
     n = lib().rexsc_profile_end(buf, max_records)
     return {buf[i].name.decode(): dict(calls=buf[i].calls, total_ms=buf[i].total_ms, total_work=buf[i].total_work)
             for i in range(n)}
+
+
+def valu_probe(mode=0, iters=2000, stream=None):
+    """-> lane-ops/s sustained by the register-only AND/popcount (mode 0) or AND-OR (mode 1) probe kernel."""
+    ms, ops = ctypes.c_double(), ctypes.c_double()
+    check(lib().rexsc_valu_probe(int(mode), int(iters), stream, ctypes.byref(ms), ctypes.byref(ops)), "rexsc_valu_probe")
+    return ops.value / (ms.value * 1e-3)

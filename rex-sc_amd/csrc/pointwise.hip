@@ -748,6 +748,7 @@ extern "C" int rexsc_split_weight(const float *w, float *w2, size_t out_channels
     if (n == 0) return REXSC_OK;
     REXSC_CHECK_ARG(w && w2, "null pointer");
     REXSC_CHECK_ARG(in_channels * taps < (1ull << 32) && n < (1ull << 31) * PW_THREADS, "tensor too large");
+    ProfScope prof("split_weight", 12.0 * n, stream);
     hipLaunchKernelGGL(split_weight_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS), 0,
                        stream, w, w2, n, (unsigned)in_channels, (unsigned)taps, w_channels_last, w2_channels_last);
     REXSC_CHECK_HIP(hipGetLastError());
@@ -763,6 +764,7 @@ extern "C" int rexsc_merge_weight_grad(const float *dw2, const float *w, float *
     if (n == 0) return REXSC_OK;
     REXSC_CHECK_ARG(dw2 && w && dw, "null pointer");
     REXSC_CHECK_ARG(in_channels * taps < (1ull << 32) && n < (1ull << 31) * PW_THREADS, "tensor too large");
+    ProfScope prof("merge_weight_grad", 16.0 * n, stream);
     hipLaunchKernelGGL(merge_weight_grad_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS),
                        0, stream, dw2, w, dw, n, (unsigned)in_channels, (unsigned)taps, dw2_channels_last,
                        w_channels_last);

@@ -70,3 +70,83 @@ extern "C" int rexsc_profile_end(rexsc_profile_record *out, int max_records)
     g_recs.clear();
     return n;
 }
+
+// ---- integer VALU peak probe ---------------------------------------------------------------------
+// A register-only kernel issuing the instruction pair of the SC compute kernel exactly as that kernel issues
+// it (v_and_b32 with a scalar operand, s_nop 0, v_bcnt_u32_b32 with its accumulate input; mode 1:
+// v_and_or_b32, the OR-1 form) on 16 independent accumulators per lane, eight waves per SIMD, no memory
+// traffic inside the timed loop.  What it sustains is the roof the AND/popcount kernels are measured against
+// on the machine at hand.
+namespace rexsc {
+namespace {
+static __device__ uint32_t g_probe_sink[64];
+
+// operands: %0..%15 accumulators, %16 scratch, %17..%20 activation words, %21..%24 weight words (SGPRs)
+#define REXSC_PROBE_PAIR(C, A, W) \
+    "v_and_b32 %16, %" #W ", %" #A "\n\ts_nop 0\n\tv_bcnt_u32_b32 %" #C ", %16, %" #C "\n\t"
+#define REXSC_PROBE_ANDOR(C, A, W) "v_and_or_b32 %" #C ", %" #A ", %" #W ", %" #C "\n\t"
+#define REXSC_PROBE_ROW(OP, A0, A1, A2, A3)                                                        \
+    OP(0, A0, 21) OP(1, A1, 22) OP(2, A2, 23) OP(3, A3, 24) OP(4, A0, 21) OP(5, A1, 22) OP(6, A2, 23) OP(7, A3, 24)       \
+    OP(8, A0, 21) OP(9, A1, 22) OP(10, A2, 23) OP(11, A3, 24) OP(12, A0, 21) OP(13, A1, 22) OP(14, A2, 23) OP(15, A3, 24)
+#define REXSC_PROBE_BODY(OP) \
+    REXSC_PROBE_ROW(OP, 17, 18, 19, 20) REXSC_PROBE_ROW(OP, 18, 19, 20, 17) REXSC_PROBE_ROW(OP, 19, 20, 17, 18) REXSC_PROBE_ROW(OP, 20, 17, 18, 19)
+
+template <int MODE>
+__global__ __launch_bounds__(256) void valu_probe_kernel(int iters, uint32_t w0, uint32_t seed)
+{
+    uint32_t c[16], a[4];
+#pragma unroll
+    for (int i = 0; i < 16; i++) c[i] = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) a[i] = seed * (threadIdx.x + 1) + i * 0x9E3779B9u;
+    const uint32_t w1 = w0 * 3u + 1u, w2 = w0 ^ 0x55555555u, w3 = ~w0;
+    for (int it = 0; it < iters; it++) {
+        // 64 slots per iteration in ONE asm statement: between separate statements the compiler would put
+        // scalar instructions of its own, and the pair's rate depends on exactly one scalar instruction per pair
+#if defined(__HIP_DEVICE_COMPILE__)
+        uint32_t t;
+#define REXSC_PROBE_OPERANDS                                                                                          \
+    : "+v"(c[0]), "+v"(c[1]), "+v"(c[2]), "+v"(c[3]), "+v"(c[4]), "+v"(c[5]), "+v"(c[6]), "+v"(c[7]), "+v"(c[8]), "+v"(c[9]), \
+      "+v"(c[10]), "+v"(c[11]), "+v"(c[12]), "+v"(c[13]), "+v"(c[14]), "+v"(c[15]), "=&v"(t)                            \
+    : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "s"(w0), "s"(w1), "s"(w2), "s"(w3)
+        if (MODE == 0) asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_PAIR) REXSC_PROBE_OPERANDS);
+        else asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_ANDOR) REXSC_PROBE_OPERANDS);
+#endif
+    }
+    uint32_t s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; i++) s ^= c[i];
+    if (s == 0xDEADBEEFu && iters < 0) g_probe_sink[threadIdx.x & 63] = s; // keeps the chain live; never taken
+}
+} // namespace
+} // namespace rexsc
+
+extern "C" int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream_, double *ms_out, double *lane_ops_out)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG((mode == 0 || mode == 1) && iters > 0 && ms_out && lane_ops_out, "valu probe: bad arguments");
+    hipDeviceProp_t prop;
+    int dev = 0;
+    REXSC_CHECK_HIP(hipGetDevice(&dev));
+    REXSC_CHECK_HIP(hipGetDeviceProperties(&prop, dev));
+    const int blocks = prop.multiProcessorCount * 8; // 4 waves per block: 8 waves per SIMD
+    hipEvent_t e0, e1;
+    REXSC_CHECK_HIP(hipEventCreate(&e0));
+    REXSC_CHECK_HIP(hipEventCreate(&e1));
+    for (int rep = 0; rep < 2; rep++) { // the first launch warms the clocks up
+        REXSC_CHECK_HIP(hipEventRecord(e0, stream));
+        if (mode == 0) hipLaunchKernelGGL(valu_probe_kernel<0>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u);
+        else hipLaunchKernelGGL(valu_probe_kernel<1>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u);
+        REXSC_CHECK_HIP(hipGetLastError());
+        REXSC_CHECK_HIP(hipEventRecord(e1, stream));
+        REXSC_CHECK_HIP(hipEventSynchronize(e1));
+    }
+    float ms = 0.f;
+    REXSC_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *ms_out = ms;
+    // VALU instructions per lane: 64 slots per iteration, two instructions each in mode 0, one in mode 1
+    *lane_ops_out = (double)blocks * 256.0 * (double)iters * 64.0 * (mode == 0 ? 2.0 : 1.0);
+    return REXSC_OK;
+}

@@ -124,7 +124,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     if (!pl.tuned) pl.ZC = Z >= 4 ? 4 : (Z >= 2 ? 2 : 1);
     const int ZC = pl.ZC, ZG = ceil_div(Z, ZC);
     const int OT = sc_compute_tile_ot();
-    const int O_pad = (int)align_up((size_t)O, (size_t)OT);
+    const int O_pad = (int)align_up((size_t)O, (size_t)16); // the weight generator works on groups of 16 output channels
     // CPU-extension rule: the and_2 generator steps the zero-including LFSR (sc_conv.cpp:365-425).  The CUDA
     // kernels have no such variant: with xnor they step the XNOR LFSR for every gen_config, seeds lowered by
     // one (sc_cuda_conv.cu:28,55-56,139), and keep seeds and operands in int8 (sc_cuda_conv.cu:37-40), which
@@ -167,6 +167,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     cp.nn = (uint32_t)n_sat | ((uint32_t)n_sat << 16);
     cp.mode = (linear && bin_config < 0) ? 1 : 0;
     cp.out_channels_last = linear ? 1 : act_cl; // linear output is [B][O]
+    cp.ot = OT;
 
     // tiling.  A block is NS waves sharing one tile of 64*px pixels x OT channels, each wave taking
     // 1/NS of the stream slots (partials meet in LDS).  Two pixels per lane halve the scalar weight

@@ -22,6 +22,7 @@ struct ComputeParams {
     int out_channels_last;
     int px;           // pixels per lane (1 or 2)
     int ns;           // waves per block; they split the slots of the block among themselves
+    int ot;           // output channels per block tile (8 or 16)
     int m_tiles, o_tiles; // filled by the launcher
     int vec_out;          // filled by the launcher: channels-last results may leave as 8-byte stores
 };

@@ -18,6 +18,7 @@
 //                     and 3 resident waves each, whole-reduction waves would quantise badly.
 //   grid            = pixel tiles x output-channel tiles x (optional) global slot splits, remapped
 //                     so that the blocks sharing a pixel tile run on the same XCD (shared L2).
+#include <stdlib.h>
 #include <string>
 
 #include "sc_compute.h"
@@ -72,11 +73,15 @@ constexpr int pick_group(int kwz, int ot)
 // count += popcount(a & w): v_and_b32 (weight word as the scalar operand) + v_bcnt_u32_b32 with its
 // accumulate input.  The accumulate form is spelled out because the compiler otherwise reassociates
 // chains of popcounts into popcount+popcount+add3, which costs 3 instructions per 2 words.
+// The s_nop between the two is deliberate: measured on gfx950 (register-only loops, 2 to 8 waves per SIMD),
+// a SIMD retires the pair in 6.2 cycles when the wave issues one scalar instruction per pair (v_and 2 cycles,
+// v_bcnt 4) and in 8.2 cycles when the pairs follow each other with nothing in between, whatever the order
+// of independent pairs; a two-cycle s_nop 1, or a nop after each of the two instructions, loses the gain again.
 __device__ __forceinline__ void and_popc_acc(uint32_t &count, uint32_t a, uint32_t w)
 {
     const uint32_t t = a & w;
 #if defined(__HIP_DEVICE_COMPILE__) // the host pass of hipcc parses device functions too
-    asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(count) : "v"(t));
+    asm("s_nop 0\n\tv_bcnt_u32_b32 %0, %1, %0" : "+v"(count) : "v"(t));
 #else
     count += __builtin_popcount(t);
 #endif
@@ -560,15 +565,16 @@ int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, i
     const int px = p.px;
     // saturation at one: the and-or instances (not in WIDE mode, whose sums are not packed)
     const bool or1 = !wide && (p.nn & 0xffffu) == 1u;
-#define REXSC_INST(KW_, ZC_)                                                                                      \
-    if (KW == KW_ && ZC == ZC_) {                                                                                 \
+#define REXSC_INST_OT(KW_, ZC_, OT_)                                                                              \
+    if (KW == KW_ && ZC == ZC_ && p.ot == OT_) {                                                                  \
         if (or1) {                                                                                                \
-            if (px == 2) return launch_compute<KW_, ZC_, 2, 16, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
-            return launch_compute<KW_, ZC_, 1, 16, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);      \
+            if (px == 2) return launch_compute<KW_, ZC_, 2, OT_, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
+            return launch_compute<KW_, ZC_, 1, OT_, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);     \
         }                                                                                                         \
-        if (px == 2) return launch_compute<KW_, ZC_, 2, 16, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
-        return launch_compute<KW_, ZC_, 1, 16, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);          \
+        if (px == 2) return launch_compute<KW_, ZC_, 2, OT_, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
+        return launch_compute<KW_, ZC_, 1, OT_, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);         \
     }
+#define REXSC_INST(KW_, ZC_) REXSC_INST_OT(KW_, ZC_, 16)
     if (wide) {
         REXSC_CHECK_ARG(KW == 1 && (ZC == 4 || ZC == 8), "wide accumulation is only built for 1x1 / linear shapes");
         if (ZC == 4) return launch_compute<1, 4, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
@@ -579,6 +585,7 @@ int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, i
     REXSC_INST(5, 1) REXSC_INST(5, 2)
     REXSC_INST(7, 1) REXSC_INST(7, 2)
 #undef REXSC_INST
+#undef REXSC_INST_OT
     set_error("SC compute: no kernel instance for KW=%d ZC=%d", KW, ZC);
     return REXSC_ERR_INVALID;
 }
