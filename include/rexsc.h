@@ -137,7 +137,9 @@ int rexsc_orn_backward(const float *grad_out, const float *x, float *grad_in, si
  * Replaces sc_extension_cuda.or_approx_n_forward_bias_std_both_acc / _backward_..._both_acc
  * (sc_cuda_pw.cu:863-927, 952-1011); scalar math of sc_cpu.hpp:264-404.
  * bias_coef / std_coef: 6 float32 coefficients each, device memory.
- * noise_out_pos / noise_out_neg: optional float32 [n] receiving the draws (NULL to skip).
+ * noise_out_pos / noise_out_neg: optional float32 [n] receiving the draws (NULL to skip).  When both are NULL
+ * the kernel draws ONE normal per output and scales it by sqrt(poly5_std(v_pos)^2 + poly5_std(v_neg)^2): the
+ * difference of the two independent noise terms has exactly that distribution and nothing else leaves the kernel.
  * offset_dev: optional device pointer to a uint64 added to `offset` when the kernel runs (NULL: none).
  * A call recorded into a HIP graph has its host arguments frozen; a caller that advances *offset_dev on
  * the stream after each call gets fresh noise on every replay. */

@@ -12,10 +12,15 @@
 namespace rexsc {
 
 // ---- scalar math -------------------------------------------------------------------------------
+// exp(-x) as one v_exp_f32 on x * -log2(e), the form the reference's CUDA kernels use (__expf, sc_device.cuh:396).
+// The rounding of the scaled argument costs |x| * 2^-24 relative; for the sums this path sees (0 <= x, results that
+// matter for x up to a few tens) that stays below 2e-6, inside the 1e-5 the float kernels are held to.
+__device__ __forceinline__ float exp_neg(float x) { return __expf(-x); }
+
 template <int N>
 __device__ __forceinline__ float orn_fwd(float x)
 {
-    const float e = expf(-x);
+    const float e = exp_neg(x);
     if constexpr (N == 1) return 1.f - e;
     if constexpr (N == 2) { float r = fmaf(-2.f, e, 2.f); return fmaf(-x, e, r); }
     if constexpr (N == 3) {
@@ -36,7 +41,7 @@ __device__ __forceinline__ float orn_fwd(float x)
 template <int N>
 __device__ __forceinline__ float orn_bwd(float g, float x)
 {
-    const float e = expf(-x);
+    const float e = exp_neg(x);
     if constexpr (N == 1) return e * g;
     float r = fmaf(x, e, e);
     if constexpr (N >= 3) r = fmaf(0.5f * (x * x), e, r);
@@ -72,6 +77,37 @@ __device__ __forceinline__ float bias_noise_fwd(float x, float xi, const Coef6 &
     xs = fmaf(s.c[4], x4, xs);
     xs = fmaf(s.c[5], x5, xs);
     return x + xb + xs * xi;
+}
+
+// f(xp, xi1) - f(xn, xi2) for f = bias_noise_fwd with two independent N(0,1) draws has the distribution of
+// (xp + poly_b(xp)) - (xn + poly_b(xn)) + sqrt(poly_s(xp)^2 + poly_s(xn)^2) * xi with ONE draw: the two noise terms
+// are independent zero-mean normals and only their difference leaves the kernel (sc_cuda_pw.cu:219-373 returns
+// nothing else).  Same fmaf order for the polynomials as bias_noise_fwd; with poly_s = 0 the value is the same.
+__device__ __forceinline__ float bias_noise_diff(float xp, float xn, float xi, const Coef6 &b, const Coef6 &s)
+{
+    float det[2], var = 0.f;
+    const float xv[2] = {xp, xn};
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const float x = xv[k];
+        const float x2 = x * x;
+        float xb = fmaf(b.c[1], x, b.c[0]);
+        const float x3 = x2 * x;
+        xb = fmaf(b.c[2], x2, xb);
+        const float x4 = x3 * x;
+        xb = fmaf(b.c[3], x3, xb);
+        const float x5 = x4 * x;
+        xb = fmaf(b.c[4], x4, xb);
+        xb = fmaf(b.c[5], x5, xb);
+        float xs = fmaf(s.c[1], x, s.c[0]);
+        xs = fmaf(s.c[2], x2, xs);
+        xs = fmaf(s.c[3], x3, xs);
+        xs = fmaf(s.c[4], x4, xs);
+        xs = fmaf(s.c[5], x5, xs);
+        det[k] = x + xb;
+        var = fmaf(xs, xs, var);
+    }
+    return (det[0] - det[1]) + __builtin_amdgcn_sqrtf(var) * xi; // v_sqrt_f32: 1 ulp, the noise scale needs no more
 }
 
 __device__ __forceinline__ float bias_bwd(float x, const Coef6 &b)
@@ -122,7 +158,7 @@ __device__ __forceinline__ void box_muller(uint32_t a, uint32_t b, float &z0, fl
 {
     const float u1 = (float)((a >> 8) + 1u) * 5.9604644775390625e-8f; // (0, 1]
     const float u2 = (float)(b >> 8) * 5.9604644775390625e-8f;        // [0, 1)
-    const float r = sqrtf(-2.f * __logf(u1));
+    const float r = __builtin_amdgcn_sqrtf(-2.f * __logf(u1));
     z0 = r * __builtin_amdgcn_cosf(u2); // v_cos_f32 takes revolutions
     z1 = r * __builtin_amdgcn_sinf(u2);
 }
@@ -174,7 +210,9 @@ __global__ __launch_bounds__(PW_THREADS) void orn_backward_kernel(const float *_
     if (i < n) gx[i] = orn_bwd<N>(g[i], half_input ? round_half(x[i]) : x[i]);
 }
 
-template <int N>
+// ONE: a single N(0,1) draw per output (bias_noise_diff); otherwise one draw per polarity, which the caller can
+// have written out (noise_p / noise_n)
+template <int N, bool ONE>
 __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_both_forward_kernel(
     const float *__restrict__ xp, const float *__restrict__ xn, const float *__restrict__ bc, const float *__restrict__ sc,
     float *__restrict__ y, size_t n, uint64_t seed, uint64_t offset, const uint64_t *__restrict__ offset_dev,
@@ -187,6 +225,25 @@ __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_both_forward_kernel(
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
         float zp[4], zn[4];
         normal4(seed, offset + q, 0u, zp);
+        if (ONE) {
+            if (q * 4 + 3 < n) {
+                const float4 a = reinterpret_cast<const float4 *>(xp)[q];
+                const float4 c = reinterpret_cast<const float4 *>(xn)[q];
+                float4 r;
+                r.x = bias_noise_diff(orn_fwd<N>(a.x), orn_fwd<N>(c.x), zp[0], b, s);
+                r.y = bias_noise_diff(orn_fwd<N>(a.y), orn_fwd<N>(c.y), zp[1], b, s);
+                r.z = bias_noise_diff(orn_fwd<N>(a.z), orn_fwd<N>(c.z), zp[2], b, s);
+                r.w = bias_noise_diff(orn_fwd<N>(a.w), orn_fwd<N>(c.w), zp[3], b, s);
+                reinterpret_cast<float4 *>(y)[q] = r;
+            } else {
+                for (int j = 0; j < 4; j++) {
+                    const size_t i = q * 4 + j;
+                    if (i >= n) break;
+                    y[i] = bias_noise_diff(orn_fwd<N>(xp[i]), orn_fwd<N>(xn[i]), zp[j], b, s);
+                }
+            }
+            continue;
+        }
         normal4(seed, offset + q, 1u, zn);
         if (q * 4 + 3 < n) {
             const float4 a = reinterpret_cast<const float4 *>(xp)[q];
@@ -330,17 +387,16 @@ __global__ __launch_bounds__(PW_THREADS) void orn_bias_std_pair_forward_kernel(
     const Coef6 b = load_coef(bc), s = load_coef(sc);
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
-        float zp[4], zn[4];
-        normal4(seed, offset + q, 0u, zp);
-        normal4(seed, offset + q, 1u, zn);
+        float z[4]; // one draw per output, the same stream the two-tensor kernel uses
+        normal4(seed, offset + q, 0u, z);
         const size_t off = pair_vec_offset(q, inner4);
         const float4 a = reinterpret_cast<const float4 *>(s2)[off];
         const float4 c = reinterpret_cast<const float4 *>(s2)[off + inner4];
         float4 r;
-        r.x = bias_noise_fwd(orn_fwd<N>(a.x), zp[0], b, s) - bias_noise_fwd(orn_fwd<N>(c.x), zn[0], b, s);
-        r.y = bias_noise_fwd(orn_fwd<N>(a.y), zp[1], b, s) - bias_noise_fwd(orn_fwd<N>(c.y), zn[1], b, s);
-        r.z = bias_noise_fwd(orn_fwd<N>(a.z), zp[2], b, s) - bias_noise_fwd(orn_fwd<N>(c.z), zn[2], b, s);
-        r.w = bias_noise_fwd(orn_fwd<N>(a.w), zp[3], b, s) - bias_noise_fwd(orn_fwd<N>(c.w), zn[3], b, s);
+        r.x = bias_noise_diff(orn_fwd<N>(a.x), orn_fwd<N>(c.x), z[0], b, s);
+        r.y = bias_noise_diff(orn_fwd<N>(a.y), orn_fwd<N>(c.y), z[1], b, s);
+        r.z = bias_noise_diff(orn_fwd<N>(a.z), orn_fwd<N>(c.z), z[2], b, s);
+        r.w = bias_noise_diff(orn_fwd<N>(a.w), orn_fwd<N>(c.w), z[3], b, s);
         reinterpret_cast<float4 *>(y)[q] = r;
     }
 }
@@ -583,9 +639,15 @@ extern "C" int rexsc_orn_bias_std_both_forward(const float *xp, const float *xn,
     if (n == 0) return REXSC_OK;
     const int grid = pw_grid((n + 3) / 4);
     ProfScope prof("orn_bias_std_both_forward", (12.0 + (noise_p ? 4.0 : 0.0) + (noise_n ? 4.0 : 0.0)) * n, stream);
-    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_bias_std_both_forward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0,
-                                               stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, offset_dev,
-                                               noise_p, noise_n));
+    if (noise_p || noise_n) {
+        REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL((orn_bias_std_both_forward_kernel<N, false>), dim3(grid), dim3(PW_THREADS), 0,
+                                                   stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, offset_dev,
+                                                   noise_p, noise_n));
+    } else {
+        REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL((orn_bias_std_both_forward_kernel<N, true>), dim3(grid), dim3(PW_THREADS), 0,
+                                                   stream, xp, xn, bias_coef, std_coef, y, n, seed, offset, offset_dev,
+                                                   noise_p, noise_n));
+    }
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

@@ -73,11 +73,18 @@ def test_fused_both_forward_backward(n, size):
     want = orc.or_approx_n_forward_bias_std_both(xp, xn, b, s, n, zp.cpu().numpy(), zn.cpu().numpy())
     _close(y, want, atol=4e-6)
     # same (seed, offset) -> same draws; another offset -> other draws
+    ya, _, _ = _ops.orn_bias_std_both_forward(tp, tn, tb, ts, n, seed=1234, offset=10, return_noise=True)
+    assert torch.equal(y, ya)
+    # without the noise outputs: one draw per output (the first stream's), scaled by the root of the summed variances
     y2 = _ops.orn_bias_std_both_forward(tp, tn, tb, ts, n, seed=1234, offset=10)
-    assert torch.equal(y, y2)
+    assert torch.equal(y2, _ops.orn_bias_std_both_forward(tp, tn, tb, ts, n, seed=1234, offset=10))
+    vp, vn = orc.or_approx_n_forward(xp, n).astype(np.float64), orc.or_approx_n_forward(xn, n).astype(np.float64)
+    poly = lambda c, v: sum(float(c[k]) * v ** k for k in range(6))
+    want2 = (vp + poly(b, vp)) - (vn + poly(b, vn)) + np.sqrt(poly(s, vp) ** 2 + poly(s, vn) ** 2) * zp.cpu().numpy()
+    _close(y2, want2.astype(np.float32), atol=4e-6)
     if size > 100:
         y3 = _ops.orn_bias_std_both_forward(tp, tn, tb, ts, n, seed=1234, offset=11)
-        assert not torch.equal(y, y3)
+        assert not torch.equal(y2, y3)
     # zero std coefficients: fully deterministic
     y0 = sc_extension_cuda.or_approx_n_forward_bias_std_both_acc(tp, tn, tb, torch.zeros(6, device="cuda"), n)
     want0 = orc.or_approx_n_forward_bias_std_both(xp, xn, b, np.zeros(6, np.float32), n, np.zeros(size, np.float32),
@@ -110,6 +117,38 @@ def test_noise_statistics():
     from scipy import stats
     ks = stats.kstest(zp[:200000].cpu().numpy().astype(np.float64), "norm")
     assert ks.pvalue > 1e-3
+
+
+def test_single_draw_noise_has_the_variance_of_the_two_draw_form():
+    """Without the noise outputs the fused forward draws one normal per output scaled by
+    sqrt(std(v_pos)^2 + std(v_neg)^2): per bin of (v_pos, v_neg) the result has the mean of the deterministic part
+    and the variance std_p^2 + std_n^2 of the reference's two-draw form (sc_cuda_pw.cu:219-373), and so has the
+    pair-layout kernel, which draws the same noise."""
+    import _ops
+    n = 1 << 22
+    bias = torch.tensor([0.01, -0.02, 0.004, 0.0, 0.001, 0.0], device="cuda")
+    std = torch.tensor([0.05, 0.03, -0.004, 0.0, 0.0, 0.0], device="cuda")
+    poly = lambda c, v: sum(c[k].item() * v ** k for k in range(6))
+    for xp_v, xn_v in ((0.3, 2.0), (1.5, 0.0), (3.0, 3.0)):
+        xp = torch.full((n,), xp_v, device="cuda")
+        xn = torch.full((n,), xn_v, device="cuda")
+        y = _ops.orn_bias_std_both_forward(xp, xn, bias, std, 2, seed=7, offset=0).double()
+        vp = float(orc.or_approx_n_forward(np.array([xp_v], np.float32), 2)[0])
+        vn = float(orc.or_approx_n_forward(np.array([xn_v], np.float32), 2)[0])
+        mean = (vp + poly(bias, vp)) - (vn + poly(bias, vn))
+        var = poly(std, vp) ** 2 + poly(std, vn) ** 2
+        assert abs(y.mean().item() - mean) < 4 * (var / n) ** 0.5 + 1e-6
+        assert abs(y.var().item() / var - 1) < 5e-3
+        z = (y - mean) / var ** 0.5
+        assert abs((z ** 3).mean().item()) < 1e-2 and abs((z ** 4).mean().item() - 3) < 3e-2
+        # the two-draw form (noise outputs requested) has the same moments
+        y2, _, _ = _ops.orn_bias_std_both_forward(xp, xn, bias, std, 2, seed=7, offset=0, return_noise=True)
+        assert abs(y2.double().mean().item() - mean) < 4 * (var / n) ** 0.5 + 1e-6
+        assert abs(y2.double().var().item() / var - 1) < 5e-3
+        # pair layout: same values as the two-tensor kernel, element for element
+        s2 = torch.stack((xp.view(-1, 64), xn.view(-1, 64)), dim=1).contiguous()
+        yp = _ops.orn_bias_std_pair_forward(s2.view(-1, 128), n // 64, 64, False, bias, std, 2, seed=7, offset=0)
+        assert torch.equal(yp.reshape(-1), y.float())
 
 
 def test_single_polarity_variants():
