@@ -63,6 +63,9 @@ typedef struct rexsc_conv_desc {
                                   * 1: the generator of the reference's CUDA conv kernels called with xnor = true
                                   *    (sc_cuda_conv.cu:28,55-56,139; sc_device.cuh:108-286): XNOR-feedback LFSR,
                                   *    seeds (index % (2^lb-1)) + 0, the same LFSR for gen_config 2; lb <= 7 */
+    int32_t act_fake_quant;      /* k > 0: x first goes through the layers' fake quantisation with prec = k - 1,   */
+    int32_t weight_fake_quant;   /* clamp(round(v * 2^prec), +-(2^prec - 1)) / 2^prec (QuantizeGrad's forward,      */
+                                 /* utils_functional.py:93-104, 117-123; utils_class.py:54,62); 0: operand as given */
 } rexsc_conv_desc;
 
 size_t rexsc_conv2d_workspace_bytes(const rexsc_conv_desc *d);
@@ -80,6 +83,20 @@ int rexsc_conv2d_plan_info(const rexsc_conv_desc *d, int64_t *out);
 int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const float *w,
                      int16_t *out_pos, int16_t *out_neg, int16_t *out_diff,
                      void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
+/* The same op with two optional extras for the caller conv2d_generic (utils_functional.py:1083-1317):
+ *  - out_value: float32 pos / L - neg / L in the layout of the int16 outputs -- the int16 -> float, "/ bit_length"
+ *    and "pos - neg" passes of :1181-1182, 1273-1274, 1317 done in the kernel that produces the sums (any of the
+ *    three int16 outputs may then be NULL and is not written);
+ *  - weight_streams: a caller-owned buffer of rexsc_conv2d_weight_streams_bytes() that receives the weight
+ *    bitstreams (and the generator table that goes with the descriptor).  With weight_streams_valid != 0 it
+ *    already holds them -- same descriptor, same weights -- and generation is skipped (w may then be NULL):
+ *    frozen weights (evaluation, utils_class.py:54 under no_grad) are expanded once, not per call. */
+size_t rexsc_conv2d_weight_streams_bytes(const rexsc_conv_desc *d);
+int rexsc_conv2d_orn_ex(const rexsc_conv_desc *d, const float *x, const float *w,
+                        int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, float *out_value,
+                        void *weight_streams, size_t weight_streams_bytes, int weight_streams_valid,
+                        void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
 
 /* The same op for callers that cannot allocate device memory or hand over a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the

@@ -16,7 +16,8 @@ class ConvDesc(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in (
         "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
         "bit_length", "lfsr_length", "gen_config", "bin_config",
-        "total_width", "load_width", "load_wait", "act_channels_last", "weight_channels_last", "xnor")]
+        "total_width", "load_width", "load_wait", "act_channels_last", "weight_channels_last", "xnor",
+        "act_fake_quant", "weight_fake_quant")]
 
 
 class LinearDesc(ctypes.Structure):
@@ -49,6 +50,8 @@ SIGNATURES = {
     "rexsc_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(ConvDesc)]),
     "rexsc_conv2d_plan_info": (_int, [ctypes.POINTER(ConvDesc), ctypes.POINTER(ctypes.c_int64)]),
     "rexsc_conv2d_orn": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_conv2d_weight_streams_bytes": (_sz, [ctypes.POINTER(ConvDesc)]),
+    "rexsc_conv2d_orn_ex": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _int, _vp, _sz, _vp]),
     "rexsc_conv2d_orn_noalloc": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp]),
     "rexsc_linear_workspace_bytes": (_sz, [ctypes.POINTER(LinearDesc)]),
     "rexsc_linear_orn": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

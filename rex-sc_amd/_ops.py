@@ -86,10 +86,46 @@ def _empty_out(shape, dtype, device, channels_last):
     return torch.empty(shape, dtype=dtype, device=device)
 
 
+class WeightStreamCache:
+    """Weight bitstreams of one weight tensor, kept between calls while the weights do not change (evaluation,
+    frozen layers).  The owner -- the layer that holds the parameter -- passes it to sc_conv2d together with the
+    PARAMETER whose values the streams were generated from; an entry is reused while that tensor's storage pointer and
+    version counter are unchanged (in-place updates by an optimiser bump the counter, `.data = ...` swaps the pointer)
+    and the call's descriptor (shapes, stream length, generator, ...) is the same."""
+
+    def __init__(self, max_entries=4):
+        self.entries = {}
+        self.max_entries = max_entries
+        self.hits = 0
+        self.misses = 0
+
+    def lookup(self, owner, desc_key, nbytes, device):
+        """-> (buffer, valid).  A fresh or stale entry comes back with valid = False and is then filled by the call."""
+        stamp = (owner.data_ptr(), owner._version, str(device))
+        ent = self.entries.get(desc_key)
+        if ent is not None and ent[0] == stamp and ent[1].numel() >= nbytes:
+            self.hits += 1
+            return ent[1], True
+        self.misses += 1
+        if ent is None and len(self.entries) >= self.max_entries:
+            self.entries.pop(next(iter(self.entries)))
+        buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        self.entries[desc_key] = (stamp, buf)
+        return buf, False
+
+    def clear(self):
+        self.entries.clear()
+
+
 def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
-              want_split=True, want_diff=False, xnor=False):
+              want_split=True, want_diff=False, xnor=False, want_value=False, weight_cache=None, weight_owner=None,
+              act_fake_quant=None, weight_fake_quant=None):
     """SC conv2d on the HIP path.  padding=(p0,p1): p0 pads the LAST axis, p1 axis 2, as the
-    reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2."""
+    reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2.
+    -> (pos, neg, diff) int16, plus the float32 tensor pos / L - neg / L as a fourth element when want_value.
+    weight_cache / weight_owner: a WeightStreamCache and the tensor whose pointer and version identify w's values
+    (default: w itself).  act_fake_quant / weight_fake_quant: precision of the layers' fake quantisation to apply to
+    the operand inside the generators (None: operand as given)."""
     _require_cuda(x, w)
     if x.dim() != 4 or w.dim() != 4 or x.size(1) != w.size(1):
         raise RuntimeError("conv2d: expected input [N,C,H,W] and weight [O,C,KH,KW] with equal C, got %s and %s"
@@ -98,28 +134,42 @@ def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_con
     xc, wc = _as_layout(x, cl_a), _as_layout(w, cl_w)
     N, C, H, W = xc.shape
     O, _, KH, KW = wc.shape
+    fq = lambda p: 0 if p is None else int(p) + 1
     d = _lib.ConvDesc(N, C, H, W, O, KH, KW, int(padding[1]), int(padding[0]), int(stride[0]), int(stride[1]),
                       int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
-                      int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w), int(bool(xnor)))
+                      int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w), int(bool(xnor)),
+                      fq(act_fake_quant), fq(weight_fake_quant))
     L = _lib.lib()
+    extended = want_value or weight_cache is not None
     with torch.cuda.device(x.device):
         Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
         Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
         shape = (N, O, Ho, Wo)
+        mk = lambda want, dt=torch.int16: _empty_out(shape, dt, x.device, cl_a) if want else None
         if N == 0 and Ho > 0 and Wo > 0:  # an empty batch has an empty result; nothing to launch
-            mk = lambda want: _empty_out(shape, torch.int16, x.device, cl_a) if want else None
-            return mk(want_split), mk(want_split), mk(want_diff)
+            res = (mk(want_split), mk(want_split), mk(want_diff))
+            return res + (mk(True, torch.float32),) if want_value else res
         ws_bytes = L.rexsc_conv2d_workspace_bytes(ctypes.byref(d))
         if ws_bytes == 0:
             _lib.check(-1, "rexsc_conv2d (planning)")
-        pos = _empty_out(shape, torch.int16, x.device, cl_a) if want_split else None
-        neg = _empty_out(shape, torch.int16, x.device, cl_a) if want_split else None
-        diff = _empty_out(shape, torch.int16, x.device, cl_a) if want_diff else None
+        pos, neg, diff = mk(want_split), mk(want_split), mk(want_diff)
         ws = _workspace(ws_bytes, x.device)
-        rc = L.rexsc_conv2d_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(diff),
-                                _ptr(ws), ws.numel(), _stream())
-        _lib.check(rc, "rexsc_conv2d_orn")
-    return pos, neg, diff
+        if not extended:
+            rc = L.rexsc_conv2d_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(diff),
+                                    _ptr(ws), ws.numel(), _stream())
+            _lib.check(rc, "rexsc_conv2d_orn")
+            return pos, neg, diff
+        value = mk(want_value, torch.float32)
+        wbuf, valid = None, False
+        if weight_cache is not None:
+            key = tuple(getattr(d, f[0]) for f in d._fields_)
+            wbuf, valid = weight_cache.lookup(w if weight_owner is None else weight_owner, key,
+                                              L.rexsc_conv2d_weight_streams_bytes(ctypes.byref(d)), x.device)
+        rc = L.rexsc_conv2d_orn_ex(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(diff), _ptr(value),
+                                   _ptr(wbuf), wbuf.numel() if wbuf is not None else 0, int(valid),
+                                   _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "rexsc_conv2d_orn_ex")
+    return (pos, neg, diff, value) if want_value else (pos, neg, diff)
 
 
 def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config):

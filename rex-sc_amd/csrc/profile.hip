@@ -100,6 +100,7 @@ __global__ __launch_bounds__(256) void valu_probe_kernel(int iters, uint32_t w0,
 #pragma unroll
     for (int i = 0; i < 4; i++) a[i] = seed * (threadIdx.x + 1) + i * 0x9E3779B9u;
     const uint32_t w1 = w0 * 3u + 1u, w2 = w0 ^ 0x55555555u, w3 = ~w0;
+    (void)w1; (void)w2; (void)w3; // only the device pass uses them
     for (int it = 0; it < iters; it++) {
         // 64 slots per iteration in ONE asm statement: between separate statements the compiler would put
         // scalar instructions of its own, and the pair's rate depends on exactly one scalar instruction per pair

@@ -115,6 +115,9 @@ struct GenParams {
     int legacy;
     float clamp_hi;
     float sign;                      // weights only: operand multiplied by +1 / -1 before the split into polarities
+    // k > 0: the operand first goes through the layers' fake quantisation with prec = k - 1
+    // (clamp(round(x * 2^prec), +-(2^prec - 1)) / 2^prec, utils_functional.py:93-104); 0: taken as it is
+    int fake_quant;
 };
 
 __host__ __device__ inline int slot_cycle(const GenParams &g, int s)

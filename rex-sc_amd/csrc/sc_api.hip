@@ -41,6 +41,8 @@ struct ScPlan {
     int Ho, Wo;
     // workspace (bytes)
     size_t off_w, off_a, off_part, off_tab_a, total;
+    size_t w_bytes;     // weight stream words incl. the over-read chunk
+    size_t wstream_off_tab, wstream_total; // layout of a separate weight-stream buffer: [Wst][state-plane table]
     size_t tab_a_words; // state-plane table of the bit-sliced activation generator (0: ballot generator)
 };
 
@@ -72,7 +74,7 @@ int fill_gen(GenParams &g, int lb, int acc, int scale, int n_slots, int div, int
     g.slot_div = div; g.slot_mul = mul; g.slot_mod = mod;
     g.total_width = tw; g.load_width = lw; g.load_wait = lwait;
     g.prog = 0;
-    g.seed_add = 0; g.legacy = 0; g.clamp_hi = (float)(scale - 1); g.sign = 1.f;
+    g.seed_add = 0; g.legacy = 0; g.clamp_hi = (float)(scale - 1); g.sign = 1.f; g.fake_quant = 0;
     REXSC_CHECK_ARG(lwait >= 1, "prog_load: load_wait must be >= 1 (got %d)", lwait);
     for (int t = 0; t < bit_length; t++) {
         const int sh = prog_shift(g, t);
@@ -86,7 +88,7 @@ int fill_gen(GenParams &g, int lb, int acc, int scale, int n_slots, int div, int
 // of B pixels is the batch, 1x1 kernel).
 int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int pad_h, int pad_w, int s0, int s1,
               int bit_length, int lfsr_length, int gen_config, int bin_config, int tw, int lw, int lwait,
-              int act_cl, int w_cl, bool linear, bool xnor)
+              int act_cl, int w_cl, bool linear, bool xnor, int act_fake_quant = 0, int weight_fake_quant = 0)
 {
     memset(&pl, 0, sizeof(pl));
     REXSC_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && O > 0 && KH > 0 && KW > 0, "non-positive dimension");
@@ -137,6 +139,10 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     rc = fill_gen(pl.gen_w, lb, acc, scale, n_slots, g, 1, 1, tw, lw, lwait, bit_length);
     if (rc) return rc;
     pl.gen_w.seed_add = 13; // POS_SEED == NEG_SEED (sc_cpu.hpp:10-11)
+    REXSC_CHECK_ARG(act_fake_quant >= 0 && act_fake_quant <= 17 && weight_fake_quant >= 0 && weight_fake_quant <= 17,
+                    "fake quantisation precision out of range (0..16)");
+    pl.gen_act.fake_quant = act_fake_quant;
+    pl.gen_w.fake_quant = weight_fake_quant;
 
     // batch chunking
     const size_t words_per_image_slot = (size_t)ZG * Hp * Wp * ZC;
@@ -228,6 +234,10 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     pl.off_tab_a = pl.off_part + align_up(part_bytes, WS_ALIGN);
     pl.tab_a_words = sng_act_table_words(ag, pl.gen_act);
     pl.total = pl.off_tab_a + align_up(pl.tab_a_words * 4, WS_ALIGN);
+    pl.w_bytes = w_bytes;
+    pl.wstream_off_tab = align_up(w_bytes, WS_ALIGN);
+    pl.wstream_total = pl.wstream_off_tab + align_up(pl.tab_a_words * 4, WS_ALIGN);
+    cp.inv_L = 1.0f / (float)bit_length;
     return REXSC_OK;
 }
 
@@ -236,7 +246,8 @@ int plan_conv(ScPlan &pl, const rexsc_conv_desc *d)
     REXSC_CHECK_ARG(d != nullptr, "null descriptor");
     return make_plan(pl, d->N, d->C, d->H, d->W, d->O, d->KH, d->KW, d->pad_h, d->pad_w, d->stride_h, d->stride_w,
                      d->bit_length, d->lfsr_length, d->gen_config, d->bin_config, d->total_width, d->load_width,
-                     d->load_wait, d->act_channels_last != 0, d->weight_channels_last != 0, false, d->xnor != 0);
+                     d->load_wait, d->act_channels_last != 0, d->weight_channels_last != 0, false, d->xnor != 0,
+                     d->act_fake_quant, d->weight_fake_quant);
 }
 
 int plan_linear(ScPlan &pl, const rexsc_linear_desc *d)
@@ -282,18 +293,27 @@ int static_scratch(void **out)
 }
 
 // The conv op proper: generators, compute, finalize, batch chunk by batch chunk, in `workspace`
-// (device memory of at least pl.total bytes).
+// (device memory of at least pl.total bytes).  wstreams != nullptr: the weight streams and the activation
+// generator's state-plane table live there (pl.wstream_total bytes) instead of in the workspace, and are
+// generated only when wstreams_valid is zero.
 int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
-             int16_t *out_neg, int16_t *out_diff, void *workspace, hipStream_t stream)
+             int16_t *out_neg, int16_t *out_diff, float *out_value, void *wstreams, int wstreams_valid, void *workspace,
+             hipStream_t stream)
 {
     uint8_t *ws = (uint8_t *)workspace;
     uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
     uint32_t *A = (uint32_t *)(ws + pl.off_a);
     uint32_t *part = (uint32_t *)(ws + pl.off_part);
     uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
-
-    int rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
-    if (rc) return rc;
+    if (wstreams) {
+        Wst = (uint32_t *)wstreams;
+        if (pl.tab_a_words) tab_a = (uint32_t *)((uint8_t *)wstreams + pl.wstream_off_tab);
+    }
+    int rc;
+    if (!wstreams || !wstreams_valid) {
+        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+        if (rc) return rc;
+    }
     const size_t in_image = (size_t)d->C * d->H * d->W;
     const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
     for (int n0 = 0; n0 < d->N; n0 += pl.n_chunk) {
@@ -307,16 +327,17 @@ int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const f
         int16_t *op = out_pos ? out_pos + n0 * out_image : nullptr;
         int16_t *on = out_neg ? out_neg + n0 * out_image : nullptr;
         int16_t *od = out_diff ? out_diff + n0 * out_image : nullptr;
+        float *ov = out_value ? out_value + n0 * out_image : nullptr;
         if (!pl.tuned) {
-            rc = sc_compute_generic(A, Wst, cp, pl.KW, pl.ZC, op, on, od, stream);
+            rc = sc_compute_generic(A, Wst, cp, pl.KW, pl.ZC, op, on, od, ov, stream);
             if (rc) return rc;
             continue;
         }
-        rc = sc_compute(A, Wst, cp, pl.KW, pl.ZC, false, part, op, on, od, stream);
+        rc = sc_compute(A, Wst, cp, pl.KW, pl.ZC, false, part, op, on, od, ov, stream);
         if (rc) return rc;
         if (!cp.direct) {
             cp.m_tiles = cp.o_tiles = 0;
-            rc = sc_finalize_i16(part, cp, op, on, od, stream);
+            rc = sc_finalize_i16(part, cp, op, on, od, ov, stream);
             if (rc) return rc;
         }
     }
@@ -375,7 +396,36 @@ extern "C" int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const 
         set_error("conv2d: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
         return REXSC_ERR_WORKSPACE;
     }
-    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, workspace, stream);
+    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, nullptr, nullptr, 0, workspace, stream);
+}
+
+extern "C" size_t rexsc_conv2d_weight_streams_bytes(const rexsc_conv_desc *d)
+{
+    ScPlan pl;
+    if (plan_conv(pl, d)) return 0;
+    return pl.wstream_total;
+}
+
+extern "C" int rexsc_conv2d_orn_ex(const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
+                                   int16_t *out_neg, int16_t *out_diff, float *out_value, void *weight_streams,
+                                   size_t weight_streams_bytes, int weight_streams_valid, void *workspace,
+                                   size_t workspace_bytes, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_conv(pl, d);
+    if (rc) return rc;
+    REXSC_CHECK_ARG(x && (w || (weight_streams && weight_streams_valid)), "null operand pointer");
+    REXSC_CHECK_ARG(out_pos || out_neg || out_diff || out_value, "no output pointer given");
+    if (!workspace || workspace_bytes < pl.total) {
+        set_error("conv2d: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
+        return REXSC_ERR_WORKSPACE;
+    }
+    if (weight_streams && weight_streams_bytes < pl.wstream_total) {
+        set_error("conv2d: weight-stream buffer of %zu bytes needed, %zu given", pl.wstream_total, weight_streams_bytes);
+        return REXSC_ERR_WORKSPACE;
+    }
+    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, out_value, weight_streams, weight_streams_valid, workspace, stream);
 }
 
 // Same op with the workspace taken from the library's static device array: no allocation of any kind,
@@ -400,7 +450,7 @@ extern "C" int rexsc_conv2d_orn_noalloc(const rexsc_conv_desc *d, const float *x
     if (rc) return rc;
     // Nothing in the workspace has to start at zero: the generators write every word the compute
     // kernel uses, and the finalize pass reads only partials the compute kernel has just written.
-    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, ws, stream);
+    return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, nullptr, nullptr, 0, ws, stream);
 }
 
 extern "C" size_t rexsc_linear_workspace_bytes(const rexsc_linear_desc *d)
@@ -432,7 +482,7 @@ extern "C" int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, cons
     if (rc) return rc;
     rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
     if (rc) return rc;
-    rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, stream);
+    rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, nullptr, stream);
     if (rc) return rc;
     return sc_finalize_i32(part, pl.cp, pl.wide, out_pos, out_neg, stream);
 }
@@ -480,7 +530,7 @@ extern "C" int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp,
             rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
             if (rc) return rc;
         }
-        rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, stream);
+        rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, nullptr, stream);
         if (rc) return rc;
         rc = sc_finalize_i32(part, pl.cp, pl.wide, pol == 0 ? out_pos : out_neg, nullptr, stream);
         if (rc) return rc;

@@ -114,6 +114,14 @@ __device__ __forceinline__ void compute_batch(const uint32_t (&a)[PX][KWZ], cons
         }
 }
 
+// The layer's float output from the packed 16-bit sums (pos | neg << 16): float(pos) / L - float(neg) / L with the
+// sums read as int16, as the reference converts its int16 results (utils_functional.py:1181-1182, 1273-1274, 1317).
+// inv_L is a power of two, so both products are exact.
+__device__ __forceinline__ float counts_value(uint32_t packed, float inv_L)
+{
+    return (float)(int16_t)(packed & 0xffffu) * inv_L - (float)(int16_t)(packed >> 16) * inv_L;
+}
+
 constexpr int MAX_NS = 4; // waves per block (each takes a share of the stream slots)
 // s_waitcnt immediate: lgkmcnt(0), vmcnt and expcnt left at their maxima (not waited for)
 constexpr int WAIT_LGKM0 = 0xC07F;
@@ -124,7 +132,8 @@ template <int KW, int ZC, int PX, int OT, int MODE>
 __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t *__restrict__ A,
                                                         const uint32_t *__restrict__ Wst, ComputeParams p,
                                                         uint32_t *__restrict__ part, int16_t *__restrict__ out_pos,
-                                                        int16_t *__restrict__ out_neg, int16_t *__restrict__ out_diff)
+                                                        int16_t *__restrict__ out_neg, int16_t *__restrict__ out_diff,
+                                                        float *__restrict__ out_value)
 {
     constexpr bool WIDE = MODE == 1, OR1 = MODE == 2;
     constexpr int KWZ = KW * ZC;
@@ -354,6 +363,9 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                         const uint32_t d2 = (v[2] - (v[2] >> 16)) & 0xffffu, d3 = (v[3] - (v[3] >> 16)) & 0xffffu;
                         *reinterpret_cast<uint2 *>(out_diff + idx) = make_uint2(d0 | (d1 << 16), d2 | (d3 << 16));
                     }
+                    if (out_value)
+                        *reinterpret_cast<float4 *>(out_value + idx) = make_float4(counts_value(v[0], p.inv_L), counts_value(v[1], p.inv_L),
+                                                                                   counts_value(v[2], p.inv_L), counts_value(v[3], p.inv_L));
                     continue;
                 }
 #pragma unroll
@@ -364,6 +376,7 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                     if (out_pos) out_pos[idx] = vp;
                     if (out_neg) out_neg[idx] = vn;
                     if (out_diff) out_diff[idx] = (int16_t)(vp - vn);
+                    if (out_value) out_value[idx] = counts_value(v[e], p.inv_L);
                 }
             } else if (p.out_channels_last) {
                 // partial sums of a global slot split, laid out like the final tensor so that the
@@ -399,7 +412,7 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
 template <bool WIDE, typename OutT, typename IdxT>
 __global__ __launch_bounds__(256) void sc_finalize_kernel(const uint32_t *__restrict__ part, ComputeParams p,
                                                           OutT *__restrict__ out_pos, OutT *__restrict__ out_neg,
-                                                          OutT *__restrict__ out_diff)
+                                                          OutT *__restrict__ out_diff, float *__restrict__ out_value)
 {
     const IdxT total = (IdxT)p.O * (IdxT)p.M;
     const long plane = (long)p.splits * p.O_pad * p.M;
@@ -439,6 +452,7 @@ __global__ __launch_bounds__(256) void sc_finalize_kernel(const uint32_t *__rest
         if (out_pos) out_pos[i] = vp;
         if (out_neg) out_neg[i] = vn;
         if (out_diff) out_diff[i] = (OutT)(vp - vn);
+        if (out_value) out_value[i] = (float)(int16_t)vp * p.inv_L - (float)(int16_t)vn * p.inv_L; // conv op only
     }
 }
 
@@ -446,7 +460,7 @@ __global__ __launch_bounds__(256) void sc_finalize_kernel(const uint32_t *__rest
 // four adjacent output channels (one 8-byte load per split) and writes 8 bytes per tensor.
 __global__ __launch_bounds__(256) void sc_finalize_nhwc4_kernel(const uint32_t *__restrict__ part, ComputeParams p,
                                                                 int16_t *__restrict__ out_pos, int16_t *__restrict__ out_neg,
-                                                                int16_t *__restrict__ out_diff)
+                                                                int16_t *__restrict__ out_diff, float *__restrict__ out_value)
 {
     const unsigned o4 = (unsigned)p.O / 4;
     const unsigned total = (unsigned)p.M * o4;
@@ -480,6 +494,12 @@ __global__ __launch_bounds__(256) void sc_finalize_nhwc4_kernel(const uint32_t *
             for (int e = 0; e < 4; e++) d[e] = (sp[e] - sn[e]) & 0xffffu;
             *reinterpret_cast<uint2 *>(out_diff + o_idx) = make_uint2(d[0] | (d[1] << 16), d[2] | (d[3] << 16));
         }
+        if (out_value) {
+            float f[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) f[e] = (float)(int16_t)sp[e] * p.inv_L - (float)(int16_t)sn[e] * p.inv_L;
+            *reinterpret_cast<float4 *>(out_value + o_idx) = make_float4(f[0], f[1], f[2], f[3]);
+        }
     }
 }
 
@@ -488,7 +508,7 @@ __global__ __launch_bounds__(256) void sc_compute_generic_kernel(const uint32_t 
                                                                  const uint32_t *__restrict__ Wst, ComputeParams p,
                                                                  int KW, int ZC, int16_t *__restrict__ out_pos,
                                                                  int16_t *__restrict__ out_neg,
-                                                                 int16_t *__restrict__ out_diff)
+                                                                 int16_t *__restrict__ out_diff, float *__restrict__ out_value)
 {
     const long total = (long)p.O * p.M;
     const int KWZ = KW * ZC;
@@ -517,19 +537,20 @@ __global__ __launch_bounds__(256) void sc_compute_generic_kernel(const uint32_t 
         if (out_pos) out_pos[idx] = vp;
         if (out_neg) out_neg[idx] = vn;
         if (out_diff) out_diff[idx] = (int16_t)(vp - vn);
+        if (out_value) out_value[idx] = (float)vp * p.inv_L - (float)vn * p.inv_L;
     }
 }
 
 // ---- host side ---------------------------------------------------------------------------------
 template <int KW, int ZC, int PX, int OT, int MODE>
 static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams p, uint32_t *part, int16_t *out_pos,
-                          int16_t *out_neg, int16_t *out_diff, hipStream_t stream)
+                          int16_t *out_neg, int16_t *out_diff, float *out_value, hipStream_t stream)
 {
     p.m_tiles = ceil_div(p.M, 64 * PX);
     p.o_tiles = p.O_pad / OT;
     // 8-byte stores of four adjacent int16 results need O % 4 == 0 and 8-byte aligned tensors
     p.vec_out = (p.O % 4 == 0 && ((uintptr_t)out_pos % 8) == 0 && ((uintptr_t)out_neg % 8) == 0 &&
-                 ((uintptr_t)out_diff % 8) == 0) ? 1 : 0;
+                 ((uintptr_t)out_diff % 8) == 0 && ((uintptr_t)out_value % 16) == 0) ? 1 : 0;
     REXSC_CHECK_ARG(p.ns >= 1 && p.ns <= MAX_NS, "SC compute: %d waves per block not supported", p.ns);
     const long blocks = (long)p.m_tiles * p.o_tiles * p.splits;
     REXSC_CHECK_ARG(blocks < (1L << 30), "SC compute: grid too large (%ld blocks)", blocks);
@@ -544,7 +565,7 @@ static int launch_compute(const uint32_t *A, const uint32_t *Wst, ComputeParams 
     // algorithmic lane-ops: (and + popcount-accumulate) x 2 polarities per 32-channel word
     ProfScope prof(name, 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
     hipLaunchKernelGGL((sc_compute_kernel<KW, ZC, PX, OT, MODE>), dim3(grid), dim3(64 * p.ns), 0, stream, A, Wst, p, part,
-                       out_pos, out_neg, out_diff);
+                       out_pos, out_neg, out_diff, out_value);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
@@ -560,7 +581,7 @@ bool sc_compute_has_instance(int KW, int ZC)
 }
 
 int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, int KW, int ZC, bool wide,
-               uint32_t *part, int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, hipStream_t stream)
+               uint32_t *part, int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, float *out_value, hipStream_t stream)
 {
     const int px = p.px;
     // saturation at one: the and-or instances (not in WIDE mode, whose sums are not packed)
@@ -568,17 +589,17 @@ int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, i
 #define REXSC_INST_OT(KW_, ZC_, OT_)                                                                              \
     if (KW == KW_ && ZC == ZC_ && p.ot == OT_) {                                                                  \
         if (or1) {                                                                                                \
-            if (px == 2) return launch_compute<KW_, ZC_, 2, OT_, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
-            return launch_compute<KW_, ZC_, 1, OT_, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);     \
+            if (px == 2) return launch_compute<KW_, ZC_, 2, OT_, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, out_value, stream); \
+            return launch_compute<KW_, ZC_, 1, OT_, 2>(A, Wst, p, part, out_pos, out_neg, out_diff, out_value, stream);     \
         }                                                                                                         \
-        if (px == 2) return launch_compute<KW_, ZC_, 2, OT_, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream); \
-        return launch_compute<KW_, ZC_, 1, OT_, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);         \
+        if (px == 2) return launch_compute<KW_, ZC_, 2, OT_, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, out_value, stream); \
+        return launch_compute<KW_, ZC_, 1, OT_, 0>(A, Wst, p, part, out_pos, out_neg, out_diff, out_value, stream);         \
     }
 #define REXSC_INST(KW_, ZC_) REXSC_INST_OT(KW_, ZC_, 16)
     if (wide) {
         REXSC_CHECK_ARG(KW == 1 && (ZC == 4 || ZC == 8), "wide accumulation is only built for 1x1 / linear shapes");
-        if (ZC == 4) return launch_compute<1, 4, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
-        return launch_compute<1, 8, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, stream);
+        if (ZC == 4) return launch_compute<1, 4, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, out_value, stream);
+        return launch_compute<1, 8, 1, 16, 1>(A, Wst, p, part, out_pos, out_neg, out_diff, out_value, stream);
     }
     REXSC_INST(1, 1) REXSC_INST(1, 2) REXSC_INST(1, 4) REXSC_INST(1, 8)
     REXSC_INST(3, 1) REXSC_INST(3, 2) REXSC_INST(3, 4)
@@ -591,34 +612,37 @@ int sc_compute(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, i
 }
 
 int sc_compute_generic(const uint32_t *A, const uint32_t *Wst, const ComputeParams &p, int KW, int ZC,
-                       int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, hipStream_t stream)
+                       int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, float *out_value, hipStream_t stream)
 {
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
     ProfScope prof("sc_compute_generic", 4.0 * p.M * p.O * p.KH * KW * p.Z * p.n_slots, stream);
     hipLaunchKernelGGL(sc_compute_generic_kernel, dim3(grid), dim3(256), 0, stream, A, Wst, p, KW, ZC, out_pos,
-                       out_neg, out_diff);
+                       out_neg, out_diff, out_value);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
 
 int sc_finalize_i16(const uint32_t *part, const ComputeParams &p, int16_t *out_pos, int16_t *out_neg,
-                    int16_t *out_diff, hipStream_t stream)
+                    int16_t *out_diff, float *out_value, hipStream_t stream)
 {
     const long total = (long)p.O * p.M;
     const int grid = (int)((total + 255) / 256 < 16384 ? (total + 255) / 256 : 16384);
-    ProfScope prof("sc_finalize_i16", (double)total * ((p.part_narrow ? 2.0 : 4.0) * p.splits + 4.0), stream);
-    const bool aligned8 = ((uintptr_t)out_pos % 8) == 0 && ((uintptr_t)out_neg % 8) == 0 && ((uintptr_t)out_diff % 8) == 0;
+    const double out_bytes = (out_pos ? 2.0 : 0.0) + (out_neg ? 2.0 : 0.0) + (out_diff ? 2.0 : 0.0) + (out_value ? 4.0 : 0.0);
+    ProfScope prof("sc_finalize_i16", (double)total * ((p.part_narrow ? 2.0 : 4.0) * p.splits + out_bytes), stream);
+    const bool aligned8 = ((uintptr_t)out_pos % 8) == 0 && ((uintptr_t)out_neg % 8) == 0 && ((uintptr_t)out_diff % 8) == 0 &&
+                          ((uintptr_t)out_value % 16) == 0;
     if (p.out_channels_last && p.part_narrow && p.O % 4 == 0 && aligned8 && total < (1L << 31)) {
         const long t4 = total / 4;
         const int grid4 = (int)((t4 + 255) / 256 < 16384 ? (t4 + 255) / 256 : 16384);
-        hipLaunchKernelGGL(sc_finalize_nhwc4_kernel, dim3(grid4), dim3(256), 0, stream, part, p, out_pos, out_neg, out_diff);
+        hipLaunchKernelGGL(sc_finalize_nhwc4_kernel, dim3(grid4), dim3(256), 0, stream, part, p, out_pos, out_neg, out_diff,
+                           out_value);
     } else if (total < (1L << 31))
         hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
-                           out_neg, out_diff);
+                           out_neg, out_diff, out_value);
     else
         hipLaunchKernelGGL((sc_finalize_kernel<false, int16_t, unsigned long>), dim3(grid), dim3(256), 0, stream, part, p,
-                           out_pos, out_neg, out_diff);
+                           out_pos, out_neg, out_diff, out_value);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
@@ -632,10 +656,10 @@ int sc_finalize_i32(const uint32_t *part, const ComputeParams &p, bool wide, int
     REXSC_CHECK_ARG(total < (1L << 31), "linear: too many outputs (%ld)", total);
     if (wide)
         hipLaunchKernelGGL((sc_finalize_kernel<true, int32_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
-                           out_neg, (int32_t *)nullptr);
+                           out_neg, (int32_t *)nullptr, (float *)nullptr);
     else
         hipLaunchKernelGGL((sc_finalize_kernel<false, int32_t, unsigned>), dim3(grid), dim3(256), 0, stream, part, p, out_pos,
-                           out_neg, (int32_t *)nullptr);
+                           out_neg, (int32_t *)nullptr, (float *)nullptr);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

@@ -67,6 +67,16 @@ int get_seq_tables(const SeqTable **tables, hipStream_t stream)
 }
 
 // ---- helpers -------------------------------------------------------------------------------
+// The layers' fake quantisation (utils_functional.py:93-104), folded into the load stage on request:
+// mul, round half to even, clamp, div by a power of two -- the same four float32 operations.
+__device__ __forceinline__ float fake_quantize(float v, int k)
+{
+    if (k <= 0) return v;
+    const float p2 = (float)(1 << (k - 1));
+    const float t = fminf(fmaxf(rintf(v * p2), 1.f - p2), p2 - 1.f);
+    return t / p2;
+}
+
 // x * S as the generator sees it: exact float32 product, rounded to binary16 in legacy mode
 __device__ __forceinline__ float scaled_operand(float v, float S, int legacy)
 {
@@ -194,7 +204,7 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
             v[k] = (inb && c < geo.C) ? x[(((long)n * geo.C + c) * geo.H + y) * geo.W + xx] : 0.f;
         }
 #pragma unroll
-        for (int k = 0; k < PER; k++) s_q[(wave + 4 * k) * QPITCH + lane] = (uint8_t)quant_ceil_pos(v[k], S, gp.clamp_hi, gp.legacy);
+        for (int k = 0; k < PER; k++) s_q[(wave + 4 * k) * QPITCH + lane] = (uint8_t)quant_ceil_pos(fake_quantize(v[k], gp.fake_quant), S, gp.clamp_hi, gp.legacy);
     } else {
         // lane = channel, each wave takes 16 pixels
         constexpr int PIX = ACT_TILE / 4, PASS = (CCH + 63) / 64;
@@ -218,7 +228,7 @@ __global__ __launch_bounds__(256) void sng_act_kernel(const float *__restrict__ 
 #pragma unroll
             for (int h = 0; h < PASS; h++) {
                 const int cl = h * 64 + lane;
-                if (cl < CCH) s_q[cl * QPITCH + wave + 4 * k] = (uint8_t)quant_ceil_pos(v[k][h], S, gp.clamp_hi, gp.legacy);
+                if (cl < CCH) s_q[cl * QPITCH + wave + 4 * k] = (uint8_t)quant_ceil_pos(fake_quantize(v[k][h], gp.fake_quant), S, gp.clamp_hi, gp.legacy);
             }
     }
     __syncthreads();
@@ -431,6 +441,10 @@ __global__ __launch_bounds__(256) void sng_act_sliced_kernel(const float *__rest
             const float *src = x + ((long)n * geo.C + c0) * plane + (long)y * geo.W + xx;
 #pragma unroll
             for (int cc = 0; cc < 32; cc++) v[cc] = c0 + cc < geo.C ? src[cc * plane] : 0.f;
+        }
+        if (gp.fake_quant) {
+#pragma unroll
+            for (int cc = 0; cc < 32; cc++) v[cc] = fake_quantize(v[cc], gp.fake_quant);
         }
         pack_quantised_all(R, v, S, gp.clamp_hi, gp.legacy, std::make_integer_sequence<int, 32>{});
         values_to_planes(R);
@@ -733,7 +747,7 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
 #pragma unroll
                 for (int i = 0; i < Q; i++) {
                     if (tq[i].ol >= wog) continue; // past the last task (wave-uniform)
-                    const float f = cur[i] * gp.sign;
+                    const float f = fake_quantize(cur[i], gp.fake_quant) * gp.sign;
                     const int cl = tq[i].cl, ol = tq[i].ol;
                     const int combo = combo0 + cl;
                     const int h = combo % HALVES, kx = combo / HALVES;

@@ -415,11 +415,11 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
             return out, bias_coef, std_coef
 
         def sc_forward():
+            # pos / L - neg / L (:1181-1182, 1273-1274, 1317) comes out of the kernel that produces the sums
             with torch.no_grad():
-                pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(
-                    activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
-                    (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
-                return _ops.sc_counts_to_float(pos, neg, bit_length)
+                return _ops.sc_conv2d(activation.data, weight.data, bit_length, LFSR_Length, padding, stride,
+                                      (prec_default, load_unit, load_wait_w), bin_config, gen_config, want_split=False,
+                                      xnor=_ops.honour_xnor(XNOR), want_value=True)[3]
 
         if not (torch.is_grad_enabled() and (activation.requires_grad or weight.requires_grad)):
             return sc_forward()  # inference: the surrogate only ever supplies gradients
@@ -510,6 +510,37 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     if sync_override == 2:
         return result_pos_value - result_neg_value, bias_coef, std_coef
     return result_pos_value - result_neg_value
+
+
+def conv2d_sc_inference(activation, weight, padding, stride, prec, weight_prec, weight_stream_cache=None, **kwargs):
+    """What the layer's  conv2d_generic(QuantizeGrad(x, prec), QuantizeGrad(w, weight_prec), sync=1)  returns when no
+    gradient is wanted (utils_class.py:54-74 under torch.no_grad()): only the integer SC forward runs, the float
+    surrogate exists for gradients alone.  From the UNQUANTISED operands: the fake quantisation is applied inside the
+    stream generators (no pass over the tensors of its own), the weight streams are kept in weight_stream_cache while
+    `weight` does not change, and pos / L - neg / L is written by the kernel that produces the sums.
+    Returns None when this shortcut does not cover the configuration (the caller then takes the general path)."""
+    bit_length = kwargs.get("bit_length", 128)
+    generator = kwargs.get("generator", None)
+    forward = kwargs.get("forward", "full_or")
+    if generator is None or kwargs.get("split_output", False) or kwargs.get("sync", 1) != 1:
+        return None
+    if os.environ.get("Global_Sync", "1") != "1" or Use_Approx or torch.is_autocast_enabled():
+        return None
+    if not (activation.is_cuda and weight.is_cuda and activation.dtype == torch.float32 and weight.dtype == torch.float32):
+        return None
+    if not (forward in ("full_or", "and_2") or (forward[:3] == "or_" and len(forward) == 4)):
+        return None
+    if prec is None or weight_prec is None or not (0 <= prec <= 16 and 0 <= weight_prec <= 16):
+        return None
+    _, bin_config, gen_config = _parse_forward(forward, generator)
+    if bin_config is None or gen_config is None:
+        return None
+    with torch.no_grad():
+        return _ops.sc_conv2d(activation, weight, bit_length, LFSR_Length, padding, stride,
+                              (prec_default, kwargs.get("load_unit", 8), kwargs.get("load_wait_w", 1)), bin_config,
+                              gen_config, want_split=False, xnor=_ops.honour_xnor(XNOR), want_value=True,
+                              weight_cache=weight_stream_cache, weight_owner=weight, act_fake_quant=prec,
+                              weight_fake_quant=weight_prec)[3]
 
 
 def linear_generic_sc(activation, weight, **kwargs):

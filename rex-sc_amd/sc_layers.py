@@ -4,6 +4,7 @@ import os
 import torch
 import torch.nn as nn
 
+import _ops
 import sc_functional as utils_f
 
 
@@ -30,19 +31,28 @@ class Conv2d_Add_Partial(nn.Conv2d):
         self.register_buffer("prune", torch.tensor([0.]))
         self.register_buffer("bias_coef", torch.zeros(self.run_args["order"] + 1))
         self.register_buffer("std_coef", torch.zeros(self.run_args["order"] + 1))
+        self._weight_streams = _ops.WeightStreamCache()  # not a buffer: derived data, never part of a state_dict
 
     def _fn_args(self):
         keys = ("bit_length", "generator", "forward", "load_unit", "load_wait_w", "split_output", "order", "sync")
         return {k: self.run_args[k] for k in keys}
 
     def forward(self, input):
-        input = utils_f.QuantizeGrad.apply(input, self.run_args["prec"])
-        g_in = input.size(1) // self.groups
-        g_wgt = self.weight.size(0) // self.groups
         if os.environ.get("Weight_Prec", "-1") != "-1":
             weight_prec = int(os.environ.get("Weight_Prec"))
         else:
             weight_prec = self.run_args["prec"]
+        if self.groups == 1 and self.run_args["sync"] == 1 and not torch.is_grad_enabled():
+            # evaluation: SC forward alone, quantisation folded into the generators, weight streams kept while the
+            # parameter does not change (REXSC_WEIGHT_STREAM_CACHE=0 regenerates them on every call)
+            cache = self._weight_streams if os.environ.get("REXSC_WEIGHT_STREAM_CACHE", "1") != "0" else None
+            out = utils_f.conv2d_sc_inference(input, self.weight, self.padding, self.stride, self.run_args["prec"], weight_prec,
+                                              weight_stream_cache=cache, **self._fn_args())
+            if out is not None:
+                return out
+        input = utils_f.QuantizeGrad.apply(input, self.run_args["prec"])
+        g_in = input.size(1) // self.groups
+        g_wgt = self.weight.size(0) // self.groups
         weight = utils_f.QuantizeGrad.apply(self.weight, weight_prec)
         out_list = []
         for g in range(self.groups):

@@ -1,0 +1,145 @@
+"""The extras of rexsc_conv2d_orn_ex around the SC conv (producer / consumer fusion, utils_functional.py:1154,
+1181-1182, 1273-1274; utils_class.py:54,62): float output written by the kernel that produces the sums, weight
+streams kept while the weights do not change, fake quantisation folded into the stream generators."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # N, C, H, W, O, K, stride, L, bin_config, cl_act
+    (2, 64, 14, 14, 48, 3, 1, 32, 1, True),      # direct store, vector path
+    (2, 64, 14, 14, 50, 3, 1, 32, 1, True),      # O % 4 != 0: scalar stores
+    (2, 64, 14, 14, 48, 3, 1, 32, 1, False),     # NCHW
+    (1, 512, 7, 7, 512, 3, 1, 32, 1, True),      # slot splits: finalize (narrow partials, vector path)
+    (1, 512, 7, 7, 510, 3, 1, 64, 3, False),     # finalize, generic path, NCHW
+    (1, 24, 10, 10, 20, 2, 1, 32, 1, False),     # no tuned instance: generic compute kernel
+    (1, 96, 4, 4, 4, 3, 1, 256, 51200, False),   # sums beyond int16: the float value follows the wrapped int16
+]
+
+
+def _operands(cfg, seed=0):
+    N, C, H, W, O, K, stride, L, bc, cla = cfg
+    rng = np.random.default_rng(seed + C + O)
+    dens = 1.0 if bc > 100 else min(1.0, 60.0 / (C * K * K) + 0.02)
+    x = (rng.integers(0, L, size=(N, C, H, W)) / L * (rng.uniform(size=(N, C, H, W)) < dens)).astype(np.float32)
+    w = (rng.integers(-L + 1, L, size=(O, C, K, K)) / L * (rng.uniform(size=(O, C, K, K)) < dens)).astype(np.float32)
+    if bc > 100:
+        w = np.abs(w)  # all weight on one polarity: its sums pass 32767 and wrap
+    xt = torch.from_numpy(x).cuda()
+    if cla:
+        xt = xt.contiguous(memory_format=torch.channels_last)
+    return x, w, xt, torch.from_numpy(w).cuda()
+
+
+@pytest.mark.parametrize("cfg", CASES, ids=lambda c: "_".join(str(v) for v in c))
+def test_float_output_equals_counts_over_L(cfg):
+    import _ops
+    N, C, H, W, O, K, stride, L, bc, cla = cfg
+    print("float epilogue", cfg, flush=True)
+    x, w, xt, wt = _operands(cfg)
+    args = (xt, wt, L, -1, (K // 2, K // 2), (stride, stride), (7, 8, 1), bc, 1)
+    pos, neg, diff, value = _ops.sc_conv2d(*args, want_split=True, want_diff=True, want_value=True)
+    p0, n0, d0 = _ops.sc_conv2d(*args, want_split=True, want_diff=True)
+    assert torch.equal(pos, p0) and torch.equal(neg, n0) and torch.equal(diff, d0)
+    assert value.dtype == torch.float32 and value.stride() == pos.stride()
+    assert torch.equal(value, pos.float() / L - neg.float() / L)
+    assert torch.equal(value, _ops.sc_counts_to_float(pos, neg, L))
+    # the float output alone (no int16 tensor is written)
+    only = _ops.sc_conv2d(*args, want_split=False, want_value=True)
+    assert only[0] is None and only[1] is None and only[2] is None and torch.equal(only[3], value)
+    opos, oneg = orc.conv2d_generic_general_split(x, w, L, -1, 16, (K // 2, K // 2), (stride, stride), (7, 8, 1), bc, 1,
+                                                  channels_last_activation=cla)
+    assert np.array_equal(value.cpu().numpy(), opos.astype(np.float32) / np.float32(L) - oneg.astype(np.float32) / np.float32(L))
+    if bc > 100:
+        assert int(np.abs(opos.astype(np.int32)).max()) > 0 and (opos < 0).any()  # the 16-bit sums did wrap
+
+
+def test_weight_stream_cache_reuse_and_invalidation():
+    import _ops
+    cfg = (2, 128, 14, 14, 64, 3, 1, 32, 1, True)
+    x, w, xt, wt = _operands(cfg, seed=5)
+    cache = _ops.WeightStreamCache()
+    args = (xt, wt, 32, -1, (1, 1), (1, 1), (7, 8, 1), 1, 1)
+    want = _ops.sc_conv2d(*args)
+    a = _ops.sc_conv2d(*args, weight_cache=cache)
+    assert (cache.hits, cache.misses) == (0, 1)
+    b = _ops.sc_conv2d(*args, weight_cache=cache)
+    assert (cache.hits, cache.misses) == (1, 1)
+    for r in (a, b):
+        assert torch.equal(r[0], want[0]) and torch.equal(r[1], want[1])
+    # other activations, same weights: the cached streams serve
+    x2 = torch.roll(xt, 1, 0).contiguous(memory_format=torch.channels_last)
+    c = _ops.sc_conv2d(x2, *args[1:], weight_cache=cache)
+    assert cache.hits == 2 and torch.equal(c[0], _ops.sc_conv2d(x2, *args[1:])[0])
+    # an in-place update of the weights bumps the version counter: regenerated
+    with torch.no_grad():
+        wt.mul_(-0.5)
+    d = _ops.sc_conv2d(*args, weight_cache=cache)
+    assert cache.misses == 2
+    want2 = _ops.sc_conv2d(*args)
+    assert torch.equal(d[0], want2[0]) and torch.equal(d[1], want2[1]) and not torch.equal(d[0], want[0])
+    # new storage behind the same tensor object
+    wt.data = torch.from_numpy(w).cuda()
+    e = _ops.sc_conv2d(*args, weight_cache=cache)
+    assert cache.misses == 3 and torch.equal(e[0], want[0])
+    # another batch size is another descriptor (its own entry); both stay valid
+    f = _ops.sc_conv2d(xt[:1].contiguous(memory_format=torch.channels_last), *args[1:], weight_cache=cache)
+    assert cache.misses == 4 and torch.equal(f[0], want[0][:1])
+    g = _ops.sc_conv2d(*args, weight_cache=cache)
+    assert cache.hits == 3 and torch.equal(g[0], want[0])
+
+
+@pytest.mark.parametrize("sng_mode", ["1", "2"])
+@pytest.mark.parametrize("cla", [False, True])
+def test_fake_quantisation_folded_into_the_generators(cla, sng_mode, monkeypatch):
+    import _ops
+    import sc_functional as uf
+    monkeypatch.setenv("REXSC_SNG_MODE", sng_mode)
+    g = torch.Generator().manual_seed(3)
+    x = (torch.rand(2, 40, 9, 9, generator=g) * 1.3 - 0.15).cuda()      # off-grid, below 0 and above 1
+    w = ((torch.rand(24, 40, 3, 3, generator=g) * 2.4 - 1.2) * (torch.rand(24, 40, 3, 3, generator=g) < 0.2)).cuda()
+    x[0, 0, 0, :6] = torch.tensor([0.5 / 128, 1.5 / 128, 2.5 / 128, 127.5 / 128, 1.0, -0.5 / 128])  # ties: half to even
+    if cla:
+        x = x.contiguous(memory_format=torch.channels_last)
+    for L, prec in ((32, 7), (64, 7), (32, 3)):
+        args = (L, -1, (1, 1), (1, 1), (7, 8, 1), 1, 1)
+        want = _ops.sc_conv2d(uf.quantize(x, prec), uf.quantize(w, prec), *args)
+        got = _ops.sc_conv2d(x, w, *args, act_fake_quant=prec, weight_fake_quant=prec)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        assert int(want[0].max()) > 0
+    xq = orc.quantize(x.cpu().numpy(), 7)
+    wq = orc.quantize(w.cpu().numpy(), 7)
+    opos, oneg = orc.conv2d_generic_general_split(xq, wq, 32, -1, 16, (1, 1), (1, 1), (7, 8, 1), 1, 1, channels_last_activation=cla)
+    got = _ops.sc_conv2d(x, w, 32, -1, (1, 1), (1, 1), (7, 8, 1), 1, 1, act_fake_quant=7, weight_fake_quant=7)
+    assert np.array_equal(got[0].cpu().numpy(), opos) and np.array_equal(got[1].cpu().numpy(), oneg)
+
+
+def test_layer_evaluation_path_equals_training_forward(monkeypatch):
+    from sc_layers import Conv2d_Add_Partial
+    torch.manual_seed(4)
+    layer = Conv2d_Add_Partial(32, 48, kernel_size=3, padding=1, stride=2, bias=False, forward="or_2", err=5).cuda()
+    x = (torch.rand(3, 32, 12, 12, device="cuda") * 1.2 - 0.1).contiguous(memory_format=torch.channels_last)
+    y_train = layer(x.clone().requires_grad_(True)).detach()
+    with torch.no_grad():
+        y1 = layer(x)
+        y2 = layer(x)
+    assert torch.equal(y1, y_train) and torch.equal(y2, y_train) and y1.stride() == y_train.stride()
+    assert (layer._weight_streams.hits, layer._weight_streams.misses) == (1, 1)
+    # an optimiser step changes the weights in place: the next evaluation regenerates the streams
+    opt = torch.optim.SGD(layer.parameters(), lr=0.5)
+    layer(x.clone().requires_grad_(True)).square().sum().backward()
+    opt.step()
+    with torch.no_grad():
+        y3 = layer(x)
+    assert layer._weight_streams.misses == 2
+    assert torch.equal(y3, layer(x.clone().requires_grad_(True)).detach()) and not torch.equal(y3, y1)
+    # switched off: same values, nothing cached
+    monkeypatch.setenv("REXSC_WEIGHT_STREAM_CACHE", "0")
+    with torch.no_grad():
+        y4 = layer(x)
+    assert torch.equal(y4, y3) and layer._weight_streams.misses == 2
+    assert "_weight_streams" not in layer.state_dict()
