@@ -175,28 +175,26 @@ struct Fixed8Params {
 __device__ __forceinline__ void fixed_pack_act16(const float *__restrict__ x, int8_t *__restrict__ xq16,
                                                  const Fixed8Params &p, unsigned bid)
 {
-    // one thread per (n, cb, yp, xp): 16 channels -> 16 bytes.  A block stays inside one (n, cb)
-    // plane (blocks_per_plane blocks each), so the per-thread index arithmetic is one 32-bit division.
+    // one thread per (n, cb, yp, xp), counted over the whole tensor so that small planes waste no lanes:
+    // 16 channels -> 16 bytes.  Lanes of a wave are neighbouring pixels: each of the 16 loads is coalesced.
     const unsigned plane = (unsigned)p.Hp * p.Wp;
-    const unsigned blocks_per_plane = (plane + 255) / 256;
-    const unsigned ncb = bid / blocks_per_plane, pblk = bid - ncb * blocks_per_plane;
+    const unsigned total = (unsigned)p.N * p.CB * plane; // the host checks that this fits 32 bits
+    const unsigned t = bid * 256 + threadIdx.x;
+    if (t >= total) return;
+    const unsigned ncb = t / plane, i = t - ncb * plane;
     const unsigned n = ncb / (unsigned)p.CB, cb = ncb - n * (unsigned)p.CB;
     const long in_plane = (long)p.H * p.W;
-    {
-        const unsigned i = pblk * 256 + threadIdx.x;
-        if (i >= plane) return;
-        const unsigned yp = i / (unsigned)p.Wp, xp = i - yp * (unsigned)p.Wp;
-        const int y = (int)yp - p.pad_h, xx = (int)xp - p.pad_w;
-        const bool inb = y >= 0 && y < p.H && xx >= 0 && xx < p.W;
-        const float *src = x + ((long)n * p.C + cb * 16) * in_plane + (long)y * p.W + xx;
-        float f[16];
+    const unsigned yp = i / (unsigned)p.Wp, xp = i - yp * (unsigned)p.Wp;
+    const int y = (int)yp - p.pad_h, xx = (int)xp - p.pad_w;
+    const bool inb = y >= 0 && y < p.H && xx >= 0 && xx < p.W;
+    const float *src = x + ((long)n * p.C + cb * 16) * in_plane + (long)y * p.W + xx;
+    float f[16];
 #pragma unroll
-        for (int k = 0; k < 16; k++) f[k] = (inb && (int)(cb * 16 + k) < p.C) ? src[k * in_plane] : 0.f;
-        uint32_t wds[4] = {0, 0, 0, 0};
+    for (int k = 0; k < 16; k++) f[k] = (inb && (int)(cb * 16 + k) < p.C) ? src[k * in_plane] : 0.f;
+    uint32_t wds[4] = {0, 0, 0, 0};
 #pragma unroll
-        for (int k = 0; k < 16; k++) wds[k >> 2] |= (uint32_t)(uint8_t)quant_round_pos(f[k], p.P2) << (8 * (k & 3));
-        reinterpret_cast<uint4 *>(xq16)[(long)ncb * plane + i] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
-    }
+    for (int k = 0; k < 16; k++) wds[k >> 2] |= (uint32_t)(uint8_t)quant_round_pos(f[k], p.P2) << (8 * (k & 3));
+    reinterpret_cast<uint4 *>(xq16)[t] = make_uint4(wds[0], wds[1], wds[2], wds[3]);
 }
 
 __device__ __forceinline__ void fixed_pack_w16(const float *__restrict__ w, int8_t *__restrict__ wq16,
@@ -676,8 +674,9 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         const double io_bytes = 4.0 * p.N * p.C * p.H * p.W + 4.0 * p.O * p.C * p.KH * p.KW + 4.0 * nout;
         {
             ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 16.0 * q.N * q.CB * q.Hp * q.Wp, stream);
-            const long pack_blocks = (((long)q.Hp * q.Wp + 255) / 256) * q.N * q.CB;
-            REXSC_CHECK_ARG(pack_blocks < (1L << 31) && (long)q.CB * q.O_pad * q.KH * q.KW < (1L << 31), "fixed conv2d: problem too large");
+            const long pack_threads = (long)q.Hp * q.Wp * q.N * q.CB;
+            REXSC_CHECK_ARG(pack_threads < (1L << 32) - 256 && (long)q.CB * q.O_pad * q.KH * q.KW < (1L << 31), "fixed conv2d: problem too large");
+            const long pack_blocks = (pack_threads + 255) / 256;
             const unsigned w_blocks = (unsigned)gridf((long)q.CB * q.O_pad * q.KH * q.KW);
             unsigned zero_blocks = 0;
             if (q.ksplit > 1) {
