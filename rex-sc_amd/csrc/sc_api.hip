@@ -42,6 +42,13 @@ struct ScPlan {
     // workspace (bytes)
     size_t off_w, off_a, off_part, off_tab_a, total;
     size_t w_bytes;     // weight stream words incl. the over-read chunk
+    // Tap folding (C*KH*KW <= 32): the whole receptive field of an output pixel fits one 32-bit word, so the
+    // generated streams are regrouped (one word per output pixel and slot, bit (ky*KW+kx)*C + c) and the compute
+    // kernel runs as a 1x1 layer with one word per pixel: the same popcounts from KH*KW times fewer AND/popcount pairs.
+    bool fold;
+    int fold_KH, fold_KW, fold_s0, fold_s1, fold_Hp, fold_Wp; // the generated (unfolded) geometry
+    size_t off_w2, off_a2, w2_bytes;                          // folded streams in the workspace
+    size_t wstream_off_w2;                                    // ... and in a separate weight-stream buffer
     size_t wstream_off_tab, wstream_total; // layout of a separate weight-stream buffer: [Wst][state-plane table]
     size_t tab_a_words; // state-plane table of the bit-sliced activation generator (0: ballot generator)
 };
@@ -167,9 +174,20 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     WeightGeom &wg = pl.wg;
     wg.O = O; wg.C = C; wg.KH = KH; wg.KW = KW; wg.channels_last = w_cl; wg.ZC = ZC; wg.ZG = ZG; wg.O_pad = O_pad;
 
+    // REXSC_FOLD_TAPS=0 switches tap folding off (tuning / tests)
+    const char *fold_env = getenv("REXSC_FOLD_TAPS");
+    pl.fold = !linear && C * KH * KW <= 32 && KH * KW > 1 && sc_compute_has_instance(1, 1) && !(fold_env && atoi(fold_env) == 0);
+    if (pl.fold) pl.tuned = true; // the folded problem is a 1x1 layer with one word per pixel: always an instance
+    pl.fold_KH = KH; pl.fold_KW = KW; pl.fold_s0 = s0; pl.fold_s1 = s1; pl.fold_Hp = Hp; pl.fold_Wp = Wp;
+    // geometry the compute kernel sees
+    const int cKH = pl.fold ? 1 : KH, cKW = pl.fold ? 1 : KW;
+    const int cHp = pl.fold ? Ho : Hp, cWp = pl.fold ? Wo : Wp, cs0 = pl.fold ? 1 : s0, cs1 = pl.fold ? 1 : s1;
+    const long c_slot_stride = pl.fold ? (long)n_chunk * Ho * Wo : ag.slot_stride;
+    if (pl.fold) pl.KW = 1;
+
     ComputeParams &cp = pl.cp;
-    cp.M = n_chunk * Ho * Wo; cp.HoWo = Ho * Wo; cp.Wo = Wo; cp.Hp = Hp; cp.Wp = Wp; cp.s0 = s0; cp.s1 = s1;
-    cp.KH = KH; cp.ZG = ZG; cp.Z = Z; cp.a_slot_stride = ag.slot_stride; cp.O = O; cp.O_pad = O_pad; cp.n_slots = n_slots;
+    cp.M = n_chunk * Ho * Wo; cp.HoWo = Ho * Wo; cp.Wo = Wo; cp.Hp = cHp; cp.Wp = cWp; cp.s0 = cs0; cp.s1 = cs1;
+    cp.KH = cKH; cp.ZG = ZG; cp.Z = Z; cp.a_slot_stride = c_slot_stride; cp.O = O; cp.O_pad = O_pad; cp.n_slots = n_slots;
     cp.nn = (uint32_t)n_sat | ((uint32_t)n_sat << 16);
     cp.mode = (linear && bin_config < 0) ? 1 : 0;
     cp.out_channels_last = linear ? 1 : act_cl; // linear output is [B][O]
@@ -198,7 +216,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
         const int max_splits = n_slots / cp.ns > 0 ? n_slots / cp.ns : 1;
         // saturation at one needs one and-or per word and polarity instead of and + popcount
         const double ops_per_word = (n_sat == 1 && !pl.wide) ? 2.0 : 4.0;
-        const double work1 = (double)ceil_div(n_slots, cp.ns) * KH * ZG * (ops_per_word * cp.px * OT * KW * ZC);
+        const double work1 = (double)ceil_div(n_slots, cp.ns) * cKH * ZG * (ops_per_word * cp.px * OT * cKW * ZC);
         const double overhead = tune_env("REXSC_TUNE_WAVE_OVERHEAD", 1500);
         double best = 0;
         for (int s = 1; s <= max_splits && s <= 16; s *= 2) {
@@ -237,6 +255,15 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     pl.w_bytes = w_bytes;
     pl.wstream_off_tab = align_up(w_bytes, WS_ALIGN);
     pl.wstream_total = pl.wstream_off_tab + align_up(pl.tab_a_words * 4, WS_ALIGN);
+    if (pl.fold) {
+        pl.w2_bytes = ((size_t)n_slots + 1) * O_pad * 2 * 4; // + one chunk for the prefetch over-read
+        const size_t a2_bytes = (size_t)n_slots * c_slot_stride * 4;
+        pl.off_w2 = pl.total;
+        pl.off_a2 = pl.off_w2 + align_up(pl.w2_bytes, WS_ALIGN);
+        pl.total = pl.off_a2 + align_up(a2_bytes, WS_ALIGN);
+        pl.wstream_off_w2 = pl.wstream_total;
+        pl.wstream_total += align_up(pl.w2_bytes, WS_ALIGN);
+    }
     cp.inv_L = 1.0f / (float)bit_length;
     return REXSC_OK;
 }
@@ -305,14 +332,21 @@ int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const f
     uint32_t *A = (uint32_t *)(ws + pl.off_a);
     uint32_t *part = (uint32_t *)(ws + pl.off_part);
     uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
+    uint32_t *W2 = pl.fold ? (uint32_t *)(ws + pl.off_w2) : nullptr;
+    uint32_t *A2 = pl.fold ? (uint32_t *)(ws + pl.off_a2) : nullptr;
     if (wstreams) {
         Wst = (uint32_t *)wstreams;
         if (pl.tab_a_words) tab_a = (uint32_t *)((uint8_t *)wstreams + pl.wstream_off_tab);
+        if (pl.fold) W2 = (uint32_t *)((uint8_t *)wstreams + pl.wstream_off_w2);
     }
     int rc;
     if (!wstreams || !wstreams_valid) {
         rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
         if (rc) return rc;
+        if (pl.fold) {
+            rc = fold_weight_streams(Wst, W2, pl.cp.n_slots, pl.fold_KH, pl.fold_KW, pl.wg.O_pad, d->C, stream);
+            if (rc) return rc;
+        }
     }
     const size_t in_image = (size_t)d->C * d->H * d->W;
     const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
@@ -324,16 +358,22 @@ int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const f
         cp.M = nc * pl.Ho * pl.Wo; // slot stride keeps the full-chunk value: the buffer is laid out for n_chunk images
         rc = sng_activations(x + n0 * in_image, A, tab_a, ag, pl.gen_act, stream);
         if (rc) return rc;
+        if (pl.fold) {
+            rc = fold_activation_streams(A, A2, cp.n_slots, pl.ag.slot_stride, cp.a_slot_stride, nc, pl.fold_Hp, pl.fold_Wp,
+                                         pl.Ho, pl.Wo, pl.fold_KH, pl.fold_KW, pl.fold_s0, pl.fold_s1, d->C, stream);
+            if (rc) return rc;
+        }
+        const uint32_t *Ac = pl.fold ? A2 : A, *Wc = pl.fold ? W2 : Wst;
         int16_t *op = out_pos ? out_pos + n0 * out_image : nullptr;
         int16_t *on = out_neg ? out_neg + n0 * out_image : nullptr;
         int16_t *od = out_diff ? out_diff + n0 * out_image : nullptr;
         float *ov = out_value ? out_value + n0 * out_image : nullptr;
         if (!pl.tuned) {
-            rc = sc_compute_generic(A, Wst, cp, pl.KW, pl.ZC, op, on, od, ov, stream);
+            rc = sc_compute_generic(Ac, Wc, cp, pl.KW, pl.ZC, op, on, od, ov, stream);
             if (rc) return rc;
             continue;
         }
-        rc = sc_compute(A, Wst, cp, pl.KW, pl.ZC, false, part, op, on, od, ov, stream);
+        rc = sc_compute(Ac, Wc, cp, pl.KW, pl.ZC, false, part, op, on, od, ov, stream);
         if (rc) return rc;
         if (!cp.direct) {
             cp.m_tiles = cp.o_tiles = 0;

@@ -35,4 +35,12 @@ int sng_activations(const float *x, uint32_t *A, const uint32_t *table, const Ac
 int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, uint32_t *act_table,
                 const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream);
 
+// Tap folding for layers whose whole receptive field fits one word (C*KH*KW <= 32, one 32-channel word per pixel):
+//   A2[slot][m]      = OR over taps of A[slot][n][yo*s0+ky][xo*s1+kx] << ((ky*KW+kx)*C),  m = (n, yo, xo)
+//   W2[slot][o][pol] = OR over taps of Wst[slot][ky][o][pol][kx]      << ((ky*KW+kx)*C)
+// so that popcount(A2 & W2) is the sum over the taps of popcount(A & Wst).
+int fold_activation_streams(const uint32_t *A, uint32_t *A2, int n_slots, long a_stride, long a2_stride, int N, int Hp, int Wp,
+                            int Ho, int Wo, int KH, int KW, int s0, int s1, int C, hipStream_t stream);
+int fold_weight_streams(const uint32_t *Wst, uint32_t *W2, int n_slots, int KH, int KW, int O_pad, int C, hipStream_t stream);
+
 } // namespace rexsc

@@ -924,4 +924,62 @@ int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenP
     }
 }
 
+// ---- tap folding --------------------------------------------------------------------------------
+// One thread per (output pixel, slot): lanes are neighbouring output pixels, so every tap's load is coalesced.
+__global__ __launch_bounds__(256) void fold_act_kernel(const uint32_t *__restrict__ A, uint32_t *__restrict__ A2, long a_stride,
+                                                       long a2_stride, unsigned M, int Hp, int Wp, int Ho, int Wo, int KH, int KW,
+                                                       int s0, int s1, int C)
+{
+    const unsigned m = blockIdx.x * 256 + threadIdx.x;
+    if (m >= M) return;
+    const unsigned HoWo = (unsigned)Ho * Wo;
+    const unsigned n = m / HoWo, r = m - n * HoWo;
+    const unsigned yo = r / (unsigned)Wo, xo = r - yo * (unsigned)Wo;
+    const uint32_t *src = A + (long)blockIdx.y * a_stride + ((long)n * Hp + yo * s0) * Wp + xo * s1;
+    uint32_t word = 0;
+    for (int ky = 0; ky < KH; ky++)
+        for (int kx = 0; kx < KW; kx++) word |= src[ky * Wp + kx] << ((ky * KW + kx) * C);
+    A2[(long)blockIdx.y * a2_stride + m] = word;
+}
+
+__global__ __launch_bounds__(256) void fold_weight_kernel(const uint32_t *__restrict__ Wst, uint32_t *__restrict__ W2, int n_slots,
+                                                          int KH, int KW, int O_pad, int C)
+{
+    // one thread per (slot, o, pol); Wst[slot][ky][o][pol][kx] (one word per pixel and tap)
+    const long total = (long)n_slots * O_pad * 2;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        const int pol = (int)(i & 1);
+        const long so = i >> 1;
+        const int o = (int)(so % O_pad), slot = (int)(so / O_pad);
+        uint32_t word = 0;
+        for (int ky = 0; ky < KH; ky++)
+            for (int kx = 0; kx < KW; kx++)
+                word |= Wst[((((long)slot * KH + ky) * O_pad + o) * 2 + pol) * KW + kx] << ((ky * KW + kx) * C);
+        W2[i] = word;
+    }
+}
+
+int fold_activation_streams(const uint32_t *A, uint32_t *A2, int n_slots, long a_stride, long a2_stride, int N, int Hp, int Wp,
+                            int Ho, int Wo, int KH, int KW, int s0, int s1, int C, hipStream_t stream)
+{
+    const long M = (long)N * Ho * Wo;
+    REXSC_CHECK_ARG(C * KH * KW <= 32 && M > 0 && M < (1L << 31) && n_slots <= 65535, "tap folding: shape out of range");
+    ProfScope prof("fold_act", 4.0 * n_slots * ((double)N * Hp * Wp + (double)M), stream);
+    hipLaunchKernelGGL(fold_act_kernel, dim3((unsigned)((M + 255) / 256), (unsigned)n_slots), dim3(256), 0, stream, A, A2, a_stride,
+                       a2_stride, (unsigned)M, Hp, Wp, Ho, Wo, KH, KW, s0, s1, C);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+int fold_weight_streams(const uint32_t *Wst, uint32_t *W2, int n_slots, int KH, int KW, int O_pad, int C, hipStream_t stream)
+{
+    REXSC_CHECK_ARG(C * KH * KW <= 32, "tap folding: receptive field wider than one word");
+    const long total = (long)n_slots * O_pad * 2;
+    ProfScope prof("fold_weight", 4.0 * total * (KH * KW + 1), stream);
+    const int grid = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
+    hipLaunchKernelGGL(fold_weight_kernel, dim3(grid), dim3(256), 0, stream, Wst, W2, n_slots, KH, KW, O_pad, C);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
 } // namespace rexsc

@@ -143,3 +143,55 @@ def test_layer_evaluation_path_equals_training_forward(monkeypatch):
         y4 = layer(x)
     assert torch.equal(y4, y3) and layer._weight_streams.misses == 2
     assert "_weight_streams" not in layer.state_dict()
+
+
+FOLD_CASES = [
+    # N, C, H, W, O, KH, KW, stride, pad, L, bin_config, gen, cl_act, cl_w
+    (4, 3, 32, 32, 32, 3, 3, (1, 1), (1, 1), 64, 2, 1, False, False),   # TinyConv's first layer (OR-3, 64-bit streams)
+    (2, 3, 17, 13, 20, 3, 3, (2, 1), (1, 0), 32, 1, 1, True, True),     # strides, asymmetric padding, both channels-last
+    (2, 1, 12, 12, 8, 5, 5, (1, 1), (2, 2), 32, 1, 1, False, False),    # 25 taps of one channel
+    (1, 2, 9, 9, 5, 4, 4, (1, 1), (1, 1), 16, 0, 1, False, False),      # a kernel width without an unfolded instance, OR-1
+    (2, 3, 10, 10, 12, 3, 3, (1, 1), (1, 1), 32, 1, 2, False, False),   # and_2 generator
+    (1, 8, 8, 8, 40, 2, 2, (2, 2), (0, 0), 128, 3, 1, False, False),    # exactly 32 bits
+    (3, 3, 6, 6, 4, 3, 3, (1, 1), (1, 1), 256, 51200, 1, False, False), # full_bin
+]
+
+
+@pytest.mark.parametrize("cfg", FOLD_CASES, ids=lambda c: "_".join(str(v) for v in c).replace(" ", ""))
+def test_tap_folding_is_bit_exact(cfg, monkeypatch):
+    """Layers whose receptive field fits one 32-bit word run on regrouped streams (one word per output pixel);
+    same sums as the tap-by-tap kernel and as the oracle."""
+    import ctypes
+    import _lib
+    import _ops
+    N, C, H, W, O, KH, KW, stride, pad, L, bc, gen, cla, clw = cfg
+    print("tap folding", cfg, flush=True)
+    rng = np.random.default_rng(hash(cfg) & 0xFFFF)
+    x = (rng.integers(0, L, size=(N, C, H, W)) / L).astype(np.float32)
+    w = (rng.integers(-L + 1, L, size=(O, C, KH, KW)) / L).astype(np.float32)
+    xt, wt = torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()
+    if cla:
+        xt = xt.contiguous(memory_format=torch.channels_last)
+    if clw:
+        wt = wt.contiguous(memory_format=torch.channels_last)
+    args = (xt, wt, L, -1, pad, stride, (7, 8, 1), bc, gen)
+    d = _lib.ConvDesc(N, C, H, W, O, KH, KW, pad[1], pad[0], stride[0], stride[1], L, -1, gen, bc, 7, 8, 1, int(cla), int(clw))
+    info = (ctypes.c_int64 * 16)()
+    _lib.check(_lib.lib().rexsc_conv2d_plan_info(ctypes.byref(d), info), "plan_info")
+    assert info[1] == 1 and info[0] == 1  # planned as a 1x1 layer on a tuned instance
+    pos, neg, _, value = _ops.sc_conv2d(*args, want_value=True)
+    opos, oneg = orc.conv2d_generic_general_split(x, w, L, -1, 16, pad, stride, (7, 8, 1), bc, gen,
+                                                  channels_last_activation=cla, channels_last_weight=clw)
+    assert opos.max() > 0
+    assert np.array_equal(pos.cpu().numpy(), opos) and np.array_equal(neg.cpu().numpy(), oneg)
+    assert torch.equal(value, pos.float() / L - neg.float() / L)
+    cache = _ops.WeightStreamCache()
+    for _ in range(2):  # folded weight streams are cached with the rest
+        p2 = _ops.sc_conv2d(*args, weight_cache=cache)[0]
+        assert torch.equal(p2, pos)
+    assert cache.hits == 1
+    monkeypatch.setenv("REXSC_FOLD_TAPS", "0")
+    _lib.check(_lib.lib().rexsc_conv2d_plan_info(ctypes.byref(d), info), "plan_info")
+    assert info[1] == KW
+    p0, n0, _ = _ops.sc_conv2d(*args)
+    assert torch.equal(p0, pos) and torch.equal(n0, neg)
