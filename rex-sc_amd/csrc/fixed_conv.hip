@@ -562,6 +562,228 @@ __global__ __launch_bounds__(256) void fixed_mfma_db_kernel(const int8_t *__rest
     }
 }
 
+// ---- fused 3x3 / stride 1 / padding 1 kernel ---------------------------------------------------------
+// The same contraction with the activation re-layout folded into the MFMA kernel: a block owns a tile of output
+// pixels (NI images x TH rows x all columns, at most 256 pixels) and 64 output channels, and walks over the
+// channel-block pairs.  Per pair it reads the float32 activations of the tile (with halo) straight from the NCHW
+// tensor, rounds / clamps / packs them to int8 in registers and puts them into LDS as 16-byte vectors
+// [half][padded pixel] -- the int8 copy never reaches HBM and the packing launch disappears -- and copies the
+// pair's 36 KB of packed weights (values and parities, laid out by fixed_pack_w_tiles exactly as LDS wants them).
+// Both MFMA operands then come from LDS.  One buffer per operand: several blocks share a CU, so one block's
+// loads overlap another block's MFMAs.
+struct FusedParams {
+    int N, C, H, W, O, O_pad;
+    int pairs;            // 32-channel groups, ceil(C / 32)
+    int TH, NI;           // tile: NI images x TH output rows x W columns
+    int tiles_y;          // tiles per image column (ceil(H / TH)); image groups: ceil(N / NI)
+    int o_tiles, n_items;
+    float P2;
+};
+
+// weights -> wpk[otile][pair][h][tap][val/par][o 0..63] 16-byte entries (one thread per entry pair)
+__global__ __launch_bounds__(256) void fixed_pack_w_tiles(const float *__restrict__ w, int8_t *__restrict__ wpk, int O, int C,
+                                                          int O_pad, int pairs, float P2)
+{
+    const unsigned total = (unsigned)O_pad * pairs * 2 * 9;
+    for (unsigned i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        const unsigned tap = i % 9, co = i / 9;                  // tap fastest: a thread group reads a contiguous run
+        const unsigned o = co % (unsigned)O_pad, cb = co / (unsigned)O_pad; // cb = 2 * pair + h
+        uint32_t vals[4] = {0, 0, 0, 0}, pars[4] = {0, 0, 0, 0};
+        if ((int)o < O) {
+            const float *src = w + ((long)o * C + cb * 16) * 9 + tap;
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                if ((int)(cb * 16 + k) < C) {
+                    const float f = src[(long)k * 9];
+                    const int q = quant_round_pos(f, P2) - quant_round_neg(f, P2);
+                    const int par = (q & 1) ? (q < 0 ? -1 : 1) : 0;
+                    vals[k >> 2] |= (uint32_t)(uint8_t)(int8_t)q << (8 * (k & 3));
+                    pars[k >> 2] |= (uint32_t)(uint8_t)(int8_t)par << (8 * (k & 3));
+                }
+            }
+        }
+        const unsigned otile = o / 64, ol = o % 64, pair = cb / 2, h = cb % 2;
+        const long e = ((((long)otile * pairs + pair) * 2 + h) * 9 + tap) * 2 * 64 + ol;
+        reinterpret_cast<uint4 *>(wpk)[e] = make_uint4(vals[0], vals[1], vals[2], vals[3]);
+        reinterpret_cast<uint4 *>(wpk)[e + 64] = make_uint4(pars[0], pars[1], pars[2], pars[3]);
+    }
+}
+
+constexpr int FUSED_W_ENTRIES = 2 * 9 * 2 * 64; // 16-byte entries of one (otile, pair): 36 KB
+
+// PBW: 32-pixel blocks per wave; AR: rounds of 256 (padded pixel, half) entries that cover the tile.
+// A block walks over its items (blockIdx.x, + gridDim.x, ...) and their pairs as one sequence of steps; the global
+// loads of step s + 1 are issued before the MFMAs of step s and land in registers while those run.
+template <int PBW, int AR>
+__global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__restrict__ x, const int8_t *__restrict__ wpk,
+                                                          int32_t *__restrict__ out, FusedParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_raw[];
+    v4i *s_w = reinterpret_cast<v4i *>(s_raw);       // [h][tap][val/par][o 0..63]
+    v4i *s_a = s_w + FUSED_W_ENTRIES;                // [h][padded pixel of the tile]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31, h = lane >> 5;
+    const int Wp = p.W + 2, RP = p.TH + 2;           // padded row length, padded rows per image of the tile
+    const int NPP = p.NI * RP * Wp;                  // padded pixels of the tile
+    const int TP = p.TH * p.W;                       // output pixels per image of the tile
+    const long plane = (long)p.H * p.W;
+    if ((int)blockIdx.x >= p.n_items) return;
+
+    // this thread's entries of the activation tile: image and padded row inside the tile, and the entry's byte
+    // offset from the tile's first halo element (first image, first channel of the pair, one row above and one
+    // column left of the tile) -- never negative, and 32 bits are enough: the host checks the tensor's size
+    int e_img[AR], e_row[AR];
+    uint32_t e_off[AR];
+    bool e_colok[AR];
+#pragma unroll
+    for (int a = 0; a < AR; a++) {
+        const int e = a * 256 + threadIdx.x;
+        const int hh = e >= NPP ? 1 : 0;
+        const int pp = e - hh * NPP;
+        const int i = pp / (RP * Wp), rem = pp - i * (RP * Wp);
+        const int row = rem / Wp, col = rem - row * Wp;
+        e_img[a] = e < 2 * NPP ? i : (1 << 28); // beyond the tile: never inside the batch
+        e_row[a] = row;
+        e_colok[a] = col >= 1 && col <= p.W;
+        e_off[a] = (uint32_t)((((long)i * p.C + hh * 16) * plane + (long)row * p.W + col) * 4);
+    }
+    // this lane's output pixels (one per 32-pixel block of the wave)
+    int l_img[PBW], l_row[PBW], l_col[PBW], abase[PBW];
+#pragma unroll
+    for (int pb = 0; pb < PBW; pb++) {
+        const int t = (wave + 4 * pb) * 32 + j;
+        const int i = t / TP, r = (t - i * TP) / p.W;
+        l_img[pb] = i < p.NI ? i : (1 << 28);
+        l_row[pb] = r;
+        l_col[pb] = t - i * TP - r * p.W;
+        abase[pb] = i < p.NI ? (i * RP + r) * Wp + l_col[pb] : 0;
+    }
+
+    v16i acc[2][PBW];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < PBW; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    constexpr int WR = FUSED_W_ENTRIES / 256;
+    v4i wreg[WR];
+    float freg[AR][16];
+
+    auto issue = [&](int item, int pair) {
+        const int otile = item % p.o_tiles, tile = item / p.o_tiles;
+        const int ty = tile % p.tiles_y, tg = tile / p.tiles_y;
+        const int n0 = tg * p.NI, y0 = ty * p.TH;
+        const v4i *src = reinterpret_cast<const v4i *>(wpk) + ((long)otile * p.pairs + pair) * FUSED_W_ENTRIES + threadIdx.x;
+#pragma unroll
+        for (int e = 0; e < WR; e++) wreg[e] = src[e * 256];
+        // (for the first tile this base lies one row and one element before the tensor; those entries are never loaded)
+        const char *xb = reinterpret_cast<const char *>(x) + (((long)n0 * p.C + pair * 32) * plane + (long)(y0 - 1) * p.W - 1) * 4;
+#pragma unroll
+        for (int a = 0; a < AR; a++) {
+            const int n = n0 + e_img[a], y = y0 + e_row[a] - 1;
+            const bool inb = e_colok[a] && n < p.N && y >= 0 && y < p.H;
+            const int kmax = inb ? p.C - pair * 32 - (a * 256 + (int)threadIdx.x >= NPP ? 16 : 0) : 0;
+            if (kmax >= 16) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) freg[a][k] = *reinterpret_cast<const float *>(xb + k * plane * 4 + e_off[a]);
+            } else if (kmax > 0) { // the channel tail of the last pair
+#pragma unroll
+                for (int k = 0; k < 16; k++)
+                    freg[a][k] = k < kmax ? *reinterpret_cast<const float *>(xb + k * plane * 4 + e_off[a]) : 0.f;
+            } else { // halo, or beyond the tile / the batch / the channels
+#pragma unroll
+                for (int k = 0; k < 16; k++) freg[a][k] = 0.f;
+            }
+        }
+    };
+
+    auto store_item = [&](int item) { // and clear the accumulators for the next item
+        const int otile = item % p.o_tiles, tile = item / p.o_tiles;
+        const int ty = tile % p.tiles_y, tg = tile / p.tiles_y;
+        const int n0 = tg * p.NI, y0 = ty * p.TH;
+        const bool whole = otile * 64 + 64 <= p.O;
+#pragma unroll
+        for (int pb = 0; pb < PBW; pb++) {
+            const int n = n0 + l_img[pb], y = y0 + l_row[pb];
+            if (n < p.N && y < p.H) {
+                int32_t *o0 = out + (((long)n * p.O + otile * 64 + 4 * h) * plane + (long)y * p.W + l_col[pb]);
+                if (whole) {
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) o0[(long)(a * 32 + 8 * (r / 4) + (r % 4)) * plane] = acc[a][pb][r];
+                } else {
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const int ol = a * 32 + 8 * (r / 4) + (r % 4);
+                            if (otile * 64 + 4 * h + ol < p.O) o0[(long)ol * plane] = acc[a][pb][r];
+                        }
+                }
+            }
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[a][pb][r] = 0;
+        }
+    };
+
+    int item = blockIdx.x, pair = 0, pending = -1;
+    issue(item, pair);
+    const float top = p.P2 - 1.f;
+    while (true) {
+        // operands of this step: registers -> LDS (activations rounded half to even and clamped to [0, P2 - 1] on the way:
+        // v_cvt_pk_u8_f32 rounds to nearest even, clamps below at zero and drops the byte into place)
+#pragma unroll
+        for (int e = 0; e < WR; e++) s_w[threadIdx.x + e * 256] = wreg[e];
+#pragma unroll
+        for (int a = 0; a < AR; a++) {
+            uint32_t wds[4] = {0, 0, 0, 0};
+#pragma unroll
+            for (int k = 0; k < 16; k++)
+                wds[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(fminf(freg[a][k] * p.P2, top), k & 3, wds[k >> 2]);
+            if (a * 256 + (int)threadIdx.x < 2 * NPP) s_a[a * 256 + threadIdx.x] = (v4i){(int)wds[0], (int)wds[1], (int)wds[2], (int)wds[3]};
+        }
+        __syncthreads();
+        // results of the item that ended with the previous step: stored here, before the next loads are issued, so
+        // that waiting for those loads never means waiting for younger stores
+        if (pending >= 0) store_item(pending);
+        pending = -1;
+        int nitem = item, npair = pair + 1;
+        if (npair == p.pairs) { npair = 0; nitem = item + gridDim.x; }
+        const bool more = nitem < p.n_items;
+        if (more) issue(nitem, npair);
+
+        const v4i *sw = s_w + h * (9 * 2 * 64) + j;
+        const v4i *sa = s_a + h * NPP;
+#pragma unroll
+        for (int ky = 0; ky < 3; ky++)
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++) {
+                const v4i *wt = sw + (ky * 3 + kx) * 2 * 64;
+                const v4i a0 = wt[0], a1 = wt[32], q0 = wt[64], q1 = wt[96];
+#pragma unroll
+                for (int pb = 0; pb < PBW; pb++) {
+                    const v4i b = sa[abase[pb] + ky * Wp + kx];
+                    const v4i par = b & ones;
+                    acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b, acc[0][pb], 0, 0, 0);
+                    acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b, acc[1][pb], 0, 0, 0);
+                    acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, par, acc[0][pb], 0, 0, 0);
+                    acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, par, acc[1][pb], 0, 0, 0);
+                }
+            }
+        if (pair == p.pairs - 1) pending = item;
+        if (!more) break;
+        item = nitem; pair = npair;
+        __syncthreads(); // all waves are done with this step's operands before the next ones overwrite them
+    }
+    if (pending >= 0) store_item(pending);
+}
+
 static int tune_flag(const char *name, int dflt)
 {
     const char *e = getenv(name);
@@ -577,6 +799,41 @@ static bool fixed_use_mfma(const FixedParams &p)
     const long pm = (1L << p.pin) - 1;
     const long bound = (long)p.C * p.KH * p.KW * (pm * pm + 1); // largest possible rounded sum of one polarity
     return bound < (long)p.max_value + 1 && (long)p.N * p.Ho * p.Wo < (1L << 31);
+}
+
+// Tile choice of the fused 3x3 kernel; false when the shape is not one it handles.
+static bool fused_plan(const FixedParams &p, int O_pad, FusedParams &f)
+{
+    if (p.KH != 3 || p.KW != 3 || p.s0 != 1 || p.s1 != 1 || p.pad_h != 1 || p.pad_w != 1) return false;
+    if (p.W > 256 || O_pad % 64 != 0) return false;
+    if (((long)p.N * p.C * p.H * p.W + 2L * p.W + 2) * 4 >= (1L << 32)) return false; // 32-bit byte offsets inside the activation tensor
+    f.N = p.N; f.C = p.C; f.H = p.H; f.W = p.W; f.O = p.O; f.O_pad = O_pad; f.P2 = p.P2;
+    f.pairs = ceil_div(p.C, 32);
+    f.o_tiles = O_pad / 64;
+    const int plane = p.H * p.W;
+    if (plane <= 128) {
+        // small planes: whole images, as many as fit 256 pixels while every CU still gets a block
+        f.TH = p.H;
+        f.NI = 256 / plane;
+        if (f.NI > p.N) f.NI = p.N;
+        while (f.NI > 1 && (long)ceil_div(p.N, f.NI) * f.o_tiles < 256) f.NI--;
+    } else {
+        f.NI = 1;
+        int th = 256 / p.W;
+        if (th > p.H) th = p.H;
+        if (th < 1) th = 1;
+        f.TH = th;
+        for (int t = th; 2 * t > th; t--) // a row count that divides the plane wastes no part of the last tile
+            if (p.H % t == 0) { f.TH = t; break; }
+    }
+    f.tiles_y = ceil_div(p.H, f.TH);
+    const long items = (long)ceil_div(p.N, f.NI) * f.tiles_y * f.o_tiles;
+    if (items >= (1L << 31)) return false;
+    f.n_items = (int)items;
+    const int NPP = f.NI * (f.TH + 2) * (p.W + 2);
+    if ((size_t)(FUSED_W_ENTRIES + 2 * NPP) * 16 > 64 * 1024) return false; // default LDS window
+    if (2 * NPP > 3 * 256) return false;                                    // three rounds of tile entries per thread
+    return ceil_div(f.NI * f.TH * p.W, 32) <= 8;
 }
 
 static int fixed_plan(const rexsc_fixed_desc *d, FixedParams &p, size_t &off_w, size_t &total)
@@ -672,6 +929,32 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         auto gridf = [](long n) { long b = (n + 255) / 256; return (int)(b > 16384 ? 16384 : (b ? b : 1)); };
         const size_t nout = (size_t)p.N * p.O * p.Ho * p.Wo;
         const double io_bytes = 4.0 * p.N * p.C * p.H * p.W + 4.0 * p.O * p.C * p.KH * p.KW + 4.0 * nout;
+        FusedParams fp;
+        // The single-pass kernel wins where the planes are large (the int8 copy of the activations it avoids is what
+        // the two-pass path spends its time on); on small planes with many channels its blocks are too few and too
+        // long to hide their load latency, and the two-pass path stays ahead.  REXSC_TUNE_FIXED_FUSED: 0 never, 2 wherever it can.
+        const int fused_mode = tune_flag("REXSC_TUNE_FIXED_FUSED", 1);
+        if (fused_mode && fused_plan(p, q.O_pad, fp) && (fused_mode == 2 || p.H * p.W >= 512)) {
+            {
+                ProfScope prof("fixed_pack_weights", 4.0 * p.O * p.C * 9 + 32.0 * q.O_pad * q.CB * 9, stream);
+                const long entries = (long)q.O_pad * q.CB * 9;
+                hipLaunchKernelGGL(fixed_pack_w_tiles, dim3((unsigned)gridf(entries)), dim3(256), 0, stream, w, wq16, p.O, p.C,
+                                   q.O_pad, fp.pairs, p.P2);
+                REXSC_CHECK_HIP(hipGetLastError());
+            }
+            ProfScope prof("fixed_conv_fused", io_bytes, stream);
+            const int NPP = fp.NI * (fp.TH + 2) * (fp.W + 2);
+            const size_t lds = (size_t)(FUSED_W_ENTRIES + 2 * NPP) * 16;
+            const int PBT = ceil_div(fp.NI * fp.TH * fp.W, 32);
+            const int AR = ceil_div(2 * NPP, 256);
+            const unsigned grid = (unsigned)(fp.n_items < 512 ? fp.n_items : 512);
+#define REXSC_FUSED(PBW_, AR_) hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_>), dim3(grid), dim3(256), lds, stream, x, wq16, out, fp)
+            if (PBT <= 4) { if (AR <= 2) REXSC_FUSED(1, 2); else REXSC_FUSED(1, 3); }
+            else { if (AR <= 2) REXSC_FUSED(2, 2); else REXSC_FUSED(2, 3); }
+#undef REXSC_FUSED
+            REXSC_CHECK_HIP(hipGetLastError());
+            return REXSC_OK;
+        }
         {
             ProfScope prof("fixed_pack", 4.0 * p.N * p.C * p.H * p.W + 16.0 * q.N * q.CB * q.Hp * q.Wp, stream);
             const long pack_threads = (long)q.Hp * q.Wp * q.N * q.CB;

@@ -236,6 +236,39 @@ def test_fixed_random_vs_oracle(cfg):
     assert np.array_equal(out.cpu().numpy(), want)
 
 
+FUSED_FIXED = [
+    # N, C, H, W, O: 3x3 / stride 1 / padding 1 shapes of the single-pass MFMA kernel, ragged in every direction
+    (5, 20, 7, 7, 70),      # several images per tile, batch not a multiple of the group, ragged channels and outputs
+    (3, 40, 30, 30, 64),    # row tiles that do not divide the plane
+    (2, 33, 57, 57, 10),    # wide rows: four rows per tile, three rounds of tile entries per thread
+    (1, 16, 13, 90, 64),    # two rows per tile
+    (7, 96, 14, 14, 192),   # one image per tile, three output tiles
+    (70, 8, 5, 9, 8),       # small planes, one image per tile
+    (600, 8, 5, 9, 8),      # small planes, two images per tile
+]
+
+
+@pytest.mark.parametrize("path", ["planner", "single_pass", "two_pass"])
+@pytest.mark.parametrize("cfg", FUSED_FIXED, ids=lambda c: "_".join(str(v) for v in c))
+def test_fixed_fused_shapes_and_out_of_range_operands(cfg, path, monkeypatch):
+    """Activations below zero, above one, at rounding ties and near-ties; weights likewise.  Once with the
+    library's own choice between the single-pass and the two-pass MFMA path, once with each forced."""
+    import fixed_extension_cuda
+    N, C, H, W, O = cfg
+    print("fixed fused", cfg, path, flush=True)
+    if path != "planner":
+        monkeypatch.setenv("REXSC_TUNE_FIXED_FUSED", "2" if path == "single_pass" else "0")
+    rng = np.random.default_rng(sum(cfg))
+    x = (rng.integers(-8, 80, size=(N, C, H, W)) / 64).astype(np.float32)            # [-1/8, 5/4) on the half grid
+    x += (rng.integers(-1, 2, size=x.shape) * 2.0 ** -20).astype(np.float32)         # just below / at / above
+    w = (rng.integers(-80, 80, size=(O, C, 3, 3)) / 64).astype(np.float32)
+    w += (rng.integers(-1, 2, size=w.shape) * 2.0 ** -20).astype(np.float32)
+    out = fixed_extension_cuda.conv2d_saturate_acc(_dev(x), _dev(w), 0, 5, 24, (1, 1), (1, 1))
+    want = orc.conv2d_saturate(x, w, 0, 5, 24, (1, 1), (1, 1))
+    assert out.shape == want.shape and np.abs(want).max() > 0
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
 # ---- REXSC_XNOR_MODE=cuda_ref: the generators of the reference's CUDA conv kernels ---------------------------
 XNOR_CONV = [
     # N, C, H, W, O, K, stride, L, lfsr_length, bin_config, gen, cl_act, cl_w
