@@ -84,6 +84,8 @@ def main():
                     help="run one function of bench_extra.py (e.g. pointwise, config4_fixed_conv) and exit (for profiler runs)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="run three 256 MiB device-to-device copies and exit (scales the rocprofv3 byte counters)")
+    ap.add_argument("--valu-probe", action="store_true",
+                    help="run the library's register-only VALU probe in all its modes, print the rates and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the SC path has no collectives); use --gpus 1",
@@ -109,6 +111,19 @@ def main():
         torch.cuda.synchronize()
         return 0
     _lib.check(_lib.lib().rexsc_init(None), "rexsc_init")
+    if args.valu_probe:
+        modes = {0: "v_and_b32 (SGPR operand); s_nop 0; v_bcnt_u32_b32 accumulate -- the compute kernel's pair",
+                 1: "v_and_or_b32 (SGPR operand) -- the OR-1 form",
+                 2: "v_and_b32 (SGPR operand); v_bcnt_u32_b32 accumulate -- the pair without the scalar instruction",
+                 3: "v_and_b32, vector registers only", 4: "v_bcnt_u32_b32 accumulate alone"}
+        res = {}
+        for m, text in modes.items():
+            rate = max(_lib.valu_probe(m, 2000) for _ in range(3))
+            # cycles one wave64 instruction occupies its SIMD at the nominal 2.4 GHz
+            res["mode%d" % m] = {"what": text, "Tlane_op_per_s": rate / 1e12,
+                                 "cycles_per_instruction": 256 * 4 * 64 * 2.4e9 / rate}
+        print(json.dumps({"valu_probe": res, "device": torch.cuda.get_device_name(0)}))
+        return 0
     if args.only_extra:
         import bench_extra
         fn = getattr(bench_extra, args.only_extra, None)  # a function of bench_extra.py, e.g. pointwise

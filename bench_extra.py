@@ -124,11 +124,17 @@ def config2_sc_linear(torch, dev):
         sc_only = lambda: sc_extension_cuda.linear_generic_general_acc(x, w, (7, 8, 1), L, -1, 1, 1, True, False)
         sec_sc = _time(torch, sc_only, 20, 3)
         prof = _profile(torch, sc_only, 5)
+        # evaluation: the layer under no_grad keeps its weight bitstreams while the parameter does not change
+        from sc_layers import Linear_Or
+        layer = Linear_Or(4096, 1024, bias=False, forward="or_2", err=6).to(dev)
+        layer.weight.copy_(w)
+        sec_eval = _time(torch, lambda: layer(x), 20, 3)
     sec_fb = _time(torch, fwd_bwd, 20, 3)
     mac = 256 * 4096 * 1024
     comp_ms = sum(v["ms"] for k, v in prof.items() if k.startswith("sc_compute"))
     out = {"workload": "SC linear OR-2, 64-bit streams, 256x4096 . (1024x4096)^T; backward through the float surrogate",
            "sc_forward_ms": sec_sc * 1e3, "forward_backward_ms": sec_fb * 1e3,
+           "eval_layer_forward_ms": sec_eval * 1e3,   # Linear_Or.forward: quantise input + SC op on cached weight streams + counts to float
            "bit_mac_per_s": mac * L / sec_sc, "samples_per_s_fwd_bwd": 256 / sec_fb,
            "valu_frac": mac * L * 4 / 32 / sec_sc / VALU_PEAK_LANEOPS,
            "sc_compute_valu_frac": mac * L * 4 / 32 / (comp_ms * 1e-3) / VALU_PEAK_LANEOPS if comp_ms else None,

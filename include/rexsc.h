@@ -127,6 +127,17 @@ int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, const float *w,
                      int32_t *out_pos, int32_t *out_neg,
                      void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
 
+/* rexsc_linear_orn with the weight bitstreams in a caller-owned buffer of rexsc_linear_weight_streams_bytes(d)
+ * bytes, as rexsc_conv2d_orn_ex keeps them for the conv op: weight_streams_valid != 0 promises that the buffer
+ * still holds the streams a previous call with the same descriptor and the same weight values generated; the
+ * weight generator is then skipped (w may be NULL).  The reference regenerates them on every call
+ * (sc_matmul.cpp:576-676) although its layers hold their weights fixed in evaluation (utils_class.py:54). */
+size_t rexsc_linear_weight_streams_bytes(const rexsc_linear_desc *d);
+int rexsc_linear_orn_ex(const rexsc_linear_desc *d, const float *x, const float *w,
+                        int32_t *out_pos, int32_t *out_neg,
+                        void *weight_streams, size_t weight_streams_bytes, int weight_streams_valid,
+                        void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
+
 /* The reference's legacy pure-torch simulation `linear_generic` (utils_functional.py:955-1081 with the
  * generators of :147-165, 254-272; generator 'lfsr', shared generators; what its Linear_Or layer runs,
  * utils_class.py:183-208) on the same kernels: operands q = ceil(float16(x * L)) with activations
@@ -261,7 +272,9 @@ int rexsc_profile_end(rexsc_profile_record *out, int max_records);
 /* Integer VALU peak probe (no counterpart in the reference): runs a register-only kernel that issues the SC
  * compute kernel's instruction pair (mode 0: v_and_b32 + v_bcnt_u32_b32 accumulate; mode 1: v_and_or_b32)
  * with eight waves per SIMD and returns its duration and the lane-operations it executed, so that roofline
- * fractions can be quoted against a peak measured on the machine at hand.  Synchronises the stream. */
+ * fractions can be quoted against a peak measured on the machine at hand.  Modes 2..4 time the pair without
+ * the scalar instruction the kernel puts between its halves, v_and_b32 on vector registers alone and
+ * v_bcnt_u32_b32 alone (the instruction costs the pair's roof is derived from).  Synchronises the stream. */
 int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream, double *ms_out, double *lane_ops_out);
 
 #ifdef __cplusplus

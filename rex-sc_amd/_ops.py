@@ -172,15 +172,19 @@ def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_con
     return (pos, neg, diff, value) if want_value else (pos, neg, diff)
 
 
-def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config):
+def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config, weight_cache=None, weight_owner=None,
+              weight_transform=None):
+    """SC linear on the HIP path -> (pos, neg) int32 [B,O].  weight_cache / weight_owner: a WeightStreamCache and the
+    tensor whose pointer and version identify the weight values (default: w itself); weight_transform: applied to w
+    only when the streams have to be generated (the layer's fake quantisation), and part of what the cache entry
+    stands for -- the caller keeps it the same function for one cache."""
     _require_cuda(x, w)
     if x.dim() != 2 or w.dim() != 2 or x.size(1) != w.size(1):
         raise RuntimeError("linear: expected input [B,C] and weight [O,C], got %s and %s"
                            % (tuple(x.shape), tuple(w.shape)))
     xc = x.detach().float().contiguous()
-    wc = w.detach().float().contiguous()
     B, C = xc.shape
-    O = wc.shape[0]
+    O = w.shape[0]
     d = _lib.LinearDesc(B, C, O, int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
                         int(prog_load[0]), int(prog_load[1]), int(prog_load[2]))
     L = _lib.lib()
@@ -194,9 +198,24 @@ def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config):
         pos = torch.empty((B, O), dtype=torch.int32, device=x.device)
         neg = torch.empty((B, O), dtype=torch.int32, device=x.device)
         ws = _workspace(ws_bytes, x.device)
-        rc = L.rexsc_linear_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws), ws.numel(),
-                                _stream())
-        _lib.check(rc, "rexsc_linear_orn")
+        wbuf, valid = None, False
+        if weight_cache is not None:
+            # the batch size is not part of the key: the weight streams do not depend on it
+            key = ("linear", C, O, int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
+                   tuple(int(v) for v in prog_load))
+            wbuf, valid = weight_cache.lookup(weight_owner if weight_owner is not None else w, key,
+                                              L.rexsc_linear_weight_streams_bytes(ctypes.byref(d)), x.device)
+        if not valid and weight_transform is not None:
+            w = weight_transform(w)
+        wc = w.detach().float().contiguous()
+        if wbuf is None:
+            rc = L.rexsc_linear_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws), ws.numel(),
+                                    _stream())
+            _lib.check(rc, "rexsc_linear_orn")
+        else:
+            rc = L.rexsc_linear_orn_ex(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(wbuf), wbuf.numel(),
+                                       1 if valid else 0, _ptr(ws), ws.numel(), _stream())
+            _lib.check(rc, "rexsc_linear_orn_ex")
     return pos, neg
 
 

@@ -732,7 +732,12 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         }
     };
 
-    int item = blockIdx.x, pair = 0, pending = -1;
+    // Consecutive items share their activation tile (they differ in the output-channel tile), and consecutive
+    // block ids land on different XCDs: renumber so that the blocks of one XCD (ids b, b + 8, ...) take consecutive
+    // items and the shared tile is served by that XCD's L2.  The host makes the grid a multiple of 8 when it can.
+    const int G = gridDim.x;
+    const int first = (G % 8 == 0) ? (int)(blockIdx.x % 8) * (G / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+    int item = first, pair = 0, pending = -1;
     issue(item, pair);
     const float top = p.P2 - 1.f;
     while (true) {
@@ -947,7 +952,8 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
             const size_t lds = (size_t)(FUSED_W_ENTRIES + 2 * NPP) * 16;
             const int PBT = ceil_div(fp.NI * fp.TH * fp.W, 32);
             const int AR = ceil_div(2 * NPP, 256);
-            const unsigned grid = (unsigned)(fp.n_items < 512 ? fp.n_items : 512);
+            unsigned grid = (unsigned)(fp.n_items < 512 ? fp.n_items : 512); // two blocks per CU stay resident
+            if (grid > 8) grid -= grid % 8;                                   // XCD-aware item order needs a multiple of 8
 #define REXSC_FUSED(PBW_, AR_) hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_>), dim3(grid), dim3(256), lds, stream, x, wq16, out, fp)
             if (PBT <= 4) { if (AR <= 2) REXSC_FUSED(1, 2); else REXSC_FUSED(1, 3); }
             else { if (AR <= 2) REXSC_FUSED(2, 2); else REXSC_FUSED(2, 3); }

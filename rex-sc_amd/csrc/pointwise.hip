@@ -531,28 +531,31 @@ __global__ __launch_bounds__(256) void calib_stats_kernel(const float *__restric
     __syncthreads();
     // A thread loads CAL_E elements (coalesced across the block), then walks the windows with the
     // elements in registers: per window a few VALU operations per element, one wave reduction and
-    // three LDS atomics per wave.  Partial sums of at most 64*CAL_E terms are kept in float, the
-    // running totals in double.
+    // three LDS atomics per wave.  Sum and sum of squares are carried in double from the first term on
+    // (the square of a float is exact in double), so that the variance the host forms from them as
+    // s2/n - (s1/n)^2 loses nothing to the partial sums even where the bias is much larger than the spread.
     const size_t tile = (size_t)blockDim.x * CAL_E;
     for (size_t t0 = (size_t)blockIdx.x * tile; t0 < n; t0 += (size_t)gridDim.x * tile) {
-        float act[CAL_E], err[CAL_E];
+        float act[CAL_E];
+        double err[CAL_E];
 #pragma unroll
         for (int j = 0; j < CAL_E; j++) {
             const size_t i = t0 + (size_t)j * blockDim.x + threadIdx.x;
             const bool ok = i < n;
             act[j] = ok ? a_act[i] : __builtin_nanf(""); // NaN belongs to no window
-            err[j] = ok ? a_bit[i] - act[j] : 0.f;
+            err[j] = ok ? (double)(a_bit[i] - act[j]) : 0.0;
         }
         for (int k = 0; k < n_win; k++) {
             const float lo = w.lo[k], hi = w.hi[k];
-            float c = 0.f, e = 0.f, e2 = 0.f;
+            float c = 0.f;
+            double e = 0.0, e2 = 0.0;
 #pragma unroll
             for (int j = 0; j < CAL_E; j++) {
                 const bool in = act[j] >= lo && act[j] < hi;
-                const float x = in ? err[j] : 0.f;
+                const double x = in ? err[j] : 0.0;
                 c += in ? 1.f : 0.f;
                 e += x;
-                e2 = fmaf(x, x, e2);
+                e2 = fma(x, x, e2);
             }
             if (__ballot(c > 0.f) == 0) continue; // wave-uniform
 #pragma unroll
@@ -563,8 +566,8 @@ __global__ __launch_bounds__(256) void calib_stats_kernel(const float *__restric
             }
             if ((threadIdx.x & 63) == 0) {
                 atomicAdd(&s_acc[k * 3 + 0], (double)c);
-                atomicAdd(&s_acc[k * 3 + 1], (double)e);
-                atomicAdd(&s_acc[k * 3 + 2], (double)e2);
+                atomicAdd(&s_acc[k * 3 + 1], e);
+                atomicAdd(&s_acc[k * 3 + 2], e2);
             }
         }
     }

@@ -76,7 +76,8 @@ extern "C" int rexsc_profile_end(rexsc_profile_record *out, int max_records)
 // it (v_and_b32 with a scalar operand, s_nop 0, v_bcnt_u32_b32 with its accumulate input; mode 1:
 // v_and_or_b32, the OR-1 form) on 16 independent accumulators per lane, eight waves per SIMD, no memory
 // traffic inside the timed loop.  What it sustains is the roof the AND/popcount kernels are measured against
-// on the machine at hand.
+// on the machine at hand.  Modes 2..4 document why the pair is issued that way: 2 is the pair without the
+// scalar instruction between its halves, 3 a v_and_b32 on vector registers only, 4 a v_bcnt_u32_b32 alone.
 namespace rexsc {
 namespace {
 static __device__ uint32_t g_probe_sink[64];
@@ -85,6 +86,9 @@ static __device__ uint32_t g_probe_sink[64];
 #define REXSC_PROBE_PAIR(C, A, W) \
     "v_and_b32 %16, %" #W ", %" #A "\n\ts_nop 0\n\tv_bcnt_u32_b32 %" #C ", %16, %" #C "\n\t"
 #define REXSC_PROBE_ANDOR(C, A, W) "v_and_or_b32 %" #C ", %" #A ", %" #W ", %" #C "\n\t"
+#define REXSC_PROBE_PAIR_BARE(C, A, W) "v_and_b32 %16, %" #W ", %" #A "\n\tv_bcnt_u32_b32 %" #C ", %16, %" #C "\n\t"
+#define REXSC_PROBE_AND(C, A, W) "v_and_b32 %" #C ", %" #A ", %" #C "\n\t"
+#define REXSC_PROBE_BCNT(C, A, W) "v_bcnt_u32_b32 %" #C ", %" #A ", %" #C "\n\t"
 #define REXSC_PROBE_ROW(OP, A0, A1, A2, A3)                                                        \
     OP(0, A0, 21) OP(1, A1, 22) OP(2, A2, 23) OP(3, A3, 24) OP(4, A0, 21) OP(5, A1, 22) OP(6, A2, 23) OP(7, A3, 24)       \
     OP(8, A0, 21) OP(9, A1, 22) OP(10, A2, 23) OP(11, A3, 24) OP(12, A0, 21) OP(13, A1, 22) OP(14, A2, 23) OP(15, A3, 24)
@@ -111,7 +115,10 @@ __global__ __launch_bounds__(256) void valu_probe_kernel(int iters, uint32_t w0,
       "+v"(c[10]), "+v"(c[11]), "+v"(c[12]), "+v"(c[13]), "+v"(c[14]), "+v"(c[15]), "=&v"(t)                            \
     : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "s"(w0), "s"(w1), "s"(w2), "s"(w3)
         if (MODE == 0) asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_PAIR) REXSC_PROBE_OPERANDS);
-        else asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_ANDOR) REXSC_PROBE_OPERANDS);
+        else if (MODE == 1) asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_ANDOR) REXSC_PROBE_OPERANDS);
+        else if (MODE == 2) asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_PAIR_BARE) REXSC_PROBE_OPERANDS);
+        else if (MODE == 3) asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_AND) REXSC_PROBE_OPERANDS);
+        else asm volatile(REXSC_PROBE_BODY(REXSC_PROBE_BCNT) REXSC_PROBE_OPERANDS);
 #endif
     }
     uint32_t s = 0;
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(256) void valu_probe_kernel(int iters, uint32_t w0,
 extern "C" int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream_, double *ms_out, double *lane_ops_out)
 {
     hipStream_t stream = (hipStream_t)stream_;
-    REXSC_CHECK_ARG((mode == 0 || mode == 1) && iters > 0 && ms_out && lane_ops_out, "valu probe: bad arguments");
+    REXSC_CHECK_ARG(mode >= 0 && mode <= 4 && iters > 0 && ms_out && lane_ops_out, "valu probe: bad arguments");
     hipDeviceProp_t prop;
     int dev = 0;
     REXSC_CHECK_HIP(hipGetDevice(&dev));
@@ -136,8 +143,13 @@ extern "C" int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream_, dou
     REXSC_CHECK_HIP(hipEventCreate(&e1));
     for (int rep = 0; rep < 2; rep++) { // the first launch warms the clocks up
         REXSC_CHECK_HIP(hipEventRecord(e0, stream));
-        if (mode == 0) hipLaunchKernelGGL(valu_probe_kernel<0>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u);
-        else hipLaunchKernelGGL(valu_probe_kernel<1>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u);
+        switch (mode) {
+        case 0: hipLaunchKernelGGL(valu_probe_kernel<0>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u); break;
+        case 1: hipLaunchKernelGGL(valu_probe_kernel<1>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u); break;
+        case 2: hipLaunchKernelGGL(valu_probe_kernel<2>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u); break;
+        case 3: hipLaunchKernelGGL(valu_probe_kernel<3>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u); break;
+        default: hipLaunchKernelGGL(valu_probe_kernel<4>, dim3(blocks), dim3(256), 0, stream, iters, 0x0F0F3355u, 12345u); break;
+        }
         REXSC_CHECK_HIP(hipGetLastError());
         REXSC_CHECK_HIP(hipEventRecord(e1, stream));
         REXSC_CHECK_HIP(hipEventSynchronize(e1));
@@ -147,7 +159,7 @@ extern "C" int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream_, dou
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     *ms_out = ms;
-    // VALU instructions per lane: 64 slots per iteration, two instructions each in mode 0, one in mode 1
-    *lane_ops_out = (double)blocks * 256.0 * (double)iters * 64.0 * (mode == 0 ? 2.0 : 1.0);
+    // VALU instructions per lane: 64 slots per iteration, two instructions each for the pairs, one otherwise
+    *lane_ops_out = (double)blocks * 256.0 * (double)iters * 64.0 * (mode == 0 || mode == 2 ? 2.0 : 1.0);
     return REXSC_OK;
 }

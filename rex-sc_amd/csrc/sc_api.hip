@@ -500,6 +500,30 @@ extern "C" size_t rexsc_linear_workspace_bytes(const rexsc_linear_desc *d)
     return pl.total;
 }
 
+static int run_linear(const ScPlan &pl, const float *x, const float *w, int32_t *out_pos, int32_t *out_neg,
+                      void *wstreams, int wstreams_valid, void *workspace, hipStream_t stream)
+{
+    uint8_t *ws = (uint8_t *)workspace;
+    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
+    uint32_t *A = (uint32_t *)(ws + pl.off_a);
+    uint32_t *part = (uint32_t *)(ws + pl.off_part);
+    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
+    if (wstreams) {
+        Wst = (uint32_t *)wstreams;
+        if (pl.tab_a_words) tab_a = (uint32_t *)((uint8_t *)wstreams + pl.wstream_off_tab);
+    }
+    int rc;
+    if (!wstreams || !wstreams_valid) {
+        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+        if (rc) return rc;
+    }
+    rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
+    if (rc) return rc;
+    rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, nullptr, stream);
+    if (rc) return rc;
+    return sc_finalize_i32(part, pl.cp, pl.wide, out_pos, out_neg, stream);
+}
+
 extern "C" int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, const float *w, int32_t *out_pos,
                                 int32_t *out_neg, void *workspace, size_t workspace_bytes, rexsc_stream_t stream_)
 {
@@ -513,18 +537,36 @@ extern "C" int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, cons
         return REXSC_ERR_WORKSPACE;
     }
     REXSC_CHECK_ARG(pl.tuned, "linear: no kernel instance for chunk width %d", pl.ZC);
-    uint8_t *ws = (uint8_t *)workspace;
-    uint32_t *Wst = (uint32_t *)(ws + pl.off_w);
-    uint32_t *A = (uint32_t *)(ws + pl.off_a);
-    uint32_t *part = (uint32_t *)(ws + pl.off_part);
-    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(ws + pl.off_tab_a) : nullptr;
-    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+    return run_linear(pl, x, w, out_pos, out_neg, nullptr, 0, workspace, stream);
+}
+
+extern "C" size_t rexsc_linear_weight_streams_bytes(const rexsc_linear_desc *d)
+{
+    ScPlan pl;
+    if (plan_linear(pl, d)) return 0;
+    return pl.wstream_total;
+}
+
+extern "C" int rexsc_linear_orn_ex(const rexsc_linear_desc *d, const float *x, const float *w, int32_t *out_pos,
+                                   int32_t *out_neg, void *weight_streams, size_t weight_streams_bytes,
+                                   int weight_streams_valid, void *workspace, size_t workspace_bytes,
+                                   rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_linear(pl, d);
     if (rc) return rc;
-    rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
-    if (rc) return rc;
-    rc = sc_compute(A, Wst, pl.cp, 1, pl.ZC, pl.wide, part, nullptr, nullptr, nullptr, nullptr, stream);
-    if (rc) return rc;
-    return sc_finalize_i32(part, pl.cp, pl.wide, out_pos, out_neg, stream);
+    REXSC_CHECK_ARG(x && out_pos && out_neg && (w || (weight_streams && weight_streams_valid)), "null pointer");
+    if (!workspace || workspace_bytes < pl.total) {
+        set_error("linear: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
+        return REXSC_ERR_WORKSPACE;
+    }
+    if (weight_streams && weight_streams_bytes < pl.wstream_total) {
+        set_error("linear: weight-stream buffer of %zu bytes needed, %zu given", pl.wstream_total, weight_streams_bytes);
+        return REXSC_ERR_WORKSPACE;
+    }
+    REXSC_CHECK_ARG(pl.tuned, "linear: no kernel instance for chunk width %d", pl.ZC);
+    return run_linear(pl, x, w, out_pos, out_neg, weight_streams, weight_streams_valid, workspace, stream);
 }
 
 // The reference's legacy pure-torch simulation `linear_generic` (utils_functional.py:955-1081; generator 'lfsr',

@@ -589,6 +589,28 @@ def linear_generic_sc(activation, weight, **kwargs):
     return pos_value - neg_value
 
 
+def linear_sc_inference(activation, weight, prec, weight_stream_cache=None, **kwargs):
+    """Forward value of Linear_Or's default path without autograd: quantise the input, run the SC linear op on the
+    quantised weights and return pos / L - neg / L.  `weight` is the layer's PARAMETER: with a weight_stream_cache
+    its bitstreams (and the quantisation pass that precedes them) are reused until the parameter changes."""
+    bit_length = setvalue_default(kwargs, "bit_length", 128)
+    forward = setvalue_default(kwargs, "forward", "or_2")
+    generator = setvalue_default(kwargs, "generator", "lfsr")
+    load_unit = setvalue_default(kwargs, "load_unit", 8)
+    load_wait_w = setvalue_default(kwargs, "load_wait_w", 1)
+    setvalue_default(kwargs, "sync", 1)
+    or_n, bin_config, gen_config = _parse_forward(forward, generator)
+    if bin_config is None or gen_config is None:
+        raise ValueError("linear_sc_inference: unsupported forward=%r / generator=%r" % (forward, generator))
+    with torch.no_grad():
+        x = quantize(activation, prec=prec)
+        pos, neg = _ops.sc_linear(x, weight, (prec_default, load_unit, load_wait_w), bit_length, LFSR_Length, bin_config,
+                                  gen_config, weight_cache=weight_stream_cache, weight_owner=weight,
+                                  weight_transform=lambda w: quantize(w, prec=prec))
+        # int16 like the CUDA op's outputs (sc_cuda.cpp:101-120), which linear_generic_sc also goes through
+        return _ops.sc_counts_to_float(pos.to(torch.int16), neg.to(torch.int16), bit_length)
+
+
 def linear_or_approx(activation, weight, true_or=False):
     """Float surrogate of OR accumulation for linear layers (utils_functional.py:600-608)."""
     if true_or:

@@ -92,13 +92,20 @@ class Linear_Or(nn.Linear):
         self.run_args["bit_length"] = 2 ** self.run_args["err"]
         super(Linear_Or, self).__init__(*kargs, **kwargs)
         self.register_buffer("weight_flag", self.weight.data.clone())
+        self._weight_streams = _ops.WeightStreamCache()
 
     def forward(self, input, prec=7, err=7, generator="lfsr"):
         if self.legacy:
             input.data = utils_f.quantize(input.data, prec=prec)
             weight = utils_f.QuantizeGrad.apply(self.weight, prec)
             return utils_f.linear_generic(input, weight, bit_length=2 ** err, forward="full_or", generator=generator)
+        keys = ("bit_length", "forward", "generator", "load_unit", "load_wait_w", "sync")
+        if self.run_args["sync"] == 1 and not torch.is_grad_enabled() and input.is_cuda:
+            # evaluation: the weight bitstreams (generated from the quantised weights) are kept while the parameter
+            # does not change (REXSC_WEIGHT_STREAM_CACHE=0 regenerates them on every call)
+            cache = self._weight_streams if os.environ.get("REXSC_WEIGHT_STREAM_CACHE", "1") != "0" else None
+            return utils_f.linear_sc_inference(input, self.weight, self.run_args["prec"], weight_stream_cache=cache,
+                                               **{k: self.run_args[k] for k in keys})
         input = utils_f.QuantizeGrad.apply(input, self.run_args["prec"])
         weight = utils_f.QuantizeGrad.apply(self.weight, self.run_args["prec"])
-        keys = ("bit_length", "forward", "generator", "load_unit", "load_wait_w", "sync")
         return utils_f.linear_generic_sc(input, weight, **{k: self.run_args[k] for k in keys})

@@ -145,6 +145,41 @@ def test_layer_evaluation_path_equals_training_forward(monkeypatch):
     assert "_weight_streams" not in layer.state_dict()
 
 
+def test_linear_layer_evaluation_path_and_weight_stream_cache(monkeypatch):
+    """Linear_Or under no_grad: same values as its training forward, weight bitstreams generated once per weight
+    version, for any batch size, and straight against the oracle on the quantised operands."""
+    import sc_functional as uf
+    from sc_layers import Linear_Or
+    torch.manual_seed(6)
+    layer = Linear_Or(96, 40, bias=False, forward="or_2", err=6).cuda()
+    with torch.no_grad():
+        layer.weight.mul_(4.0)
+    x = torch.rand(5, 96, device="cuda") * 1.1 - 0.05
+    y_train = layer(x.clone().requires_grad_(True)).detach()
+    with torch.no_grad():
+        y1 = layer(x)
+        y2 = layer(x)
+        y_small = layer(x[:2])          # another batch size shares the entry
+    assert torch.equal(y1, y_train) and torch.equal(y2, y_train) and torch.equal(y_small, y_train[:2])
+    assert (layer._weight_streams.hits, layer._weight_streams.misses) == (2, 1)
+    xq = uf.quantize(x, 7).cpu().numpy()
+    wq = uf.quantize(layer.weight.data, 7).cpu().numpy()
+    pos, neg = orc.linear_generic_general(xq, wq, (7, 8, 1), 64, -1, 1, 1, True, False)
+    assert np.array_equal(y1.cpu().numpy(), (pos.astype(np.float32) - neg.astype(np.float32)) / 64) and np.abs(pos).max() > 0
+    opt = torch.optim.SGD(layer.parameters(), lr=0.5)
+    layer(x.clone().requires_grad_(True)).square().sum().backward()
+    opt.step()
+    with torch.no_grad():
+        y3 = layer(x)
+    assert layer._weight_streams.misses == 2
+    assert torch.equal(y3, layer(x.clone().requires_grad_(True)).detach()) and not torch.equal(y3, y1)
+    monkeypatch.setenv("REXSC_WEIGHT_STREAM_CACHE", "0")
+    with torch.no_grad():
+        y4 = layer(x)
+    assert torch.equal(y4, y3) and layer._weight_streams.misses == 2
+    assert "_weight_streams" not in layer.state_dict()
+
+
 FOLD_CASES = [
     # N, C, H, W, O, KH, KW, stride, pad, L, bin_config, gen, cl_act, cl_w
     (4, 3, 32, 32, 32, 3, 3, (1, 1), (1, 1), 64, 2, 1, False, False),   # TinyConv's first layer (OR-3, 64-bit streams)

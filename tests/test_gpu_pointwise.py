@@ -187,10 +187,27 @@ def test_calib_stats_kernel():
         sel = (a_act >= lo[k]) & (a_act < hi[k])
         err = (a_bit[sel] - a_act[sel]).astype(np.float64)
         assert st[k, 0] == sel.sum()
-        # partial sums of up to 1024 terms are float32, the totals float64 (the reference works in
-        # float32 throughout): 1e-6 of the sum of magnitudes
-        assert abs(st[k, 1] - err.sum()) <= 1e-6 * np.abs(err).sum() + 1e-9
-        assert np.isclose(st[k, 2], (err * err).sum(), rtol=1e-6, atol=1e-9)
+        # sums and sums of squares are carried in float64 from the first term on (the reference works in float32
+        # throughout)
+        assert abs(st[k, 1] - err.sum()) <= 1e-12 * np.abs(err).sum() + 1e-12
+        assert np.isclose(st[k, 2], (err * err).sum(), rtol=1e-12, atol=1e-12)
+
+
+def test_calib_stats_variance_survives_a_large_bias():
+    """A spread a thousand times smaller than the bias: the variance formed from the returned sums as
+    s2/n - (s1/n)^2 still agrees with the float64 variance of the float32 errors."""
+    import _ops
+    rng = np.random.default_rng(9)
+    n = 1 << 20
+    a_act = rng.uniform(0, 1, n).astype(np.float32)
+    a_bit = (a_act + 1.0 + 1e-3 * rng.normal(size=n)).astype(np.float32)
+    st = _ops.calib_stats(torch.from_numpy(a_bit).cuda(), torch.from_numpy(a_act).cuda(), [np.float32(0)],
+                          [np.float32(2)]).cpu().numpy()
+    err = (a_bit - a_act).astype(np.float64)
+    cnt, s1, s2 = st[0]
+    assert cnt == n
+    var = s2 / cnt - (s1 / cnt) ** 2
+    assert np.isclose(var, err.var(), rtol=1e-6)
 
 
 def test_noise_stream_follows_the_torch_generator():
