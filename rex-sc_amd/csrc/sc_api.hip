@@ -199,8 +199,20 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
     // (256 CUs x 4 SIMDs x 3) so that its tail is short; what the tiles and NS do not supply comes
     // from splitting the slots over blocks as well (partials merged by the finalize kernel).
     const int o_tiles = O_pad / OT;
-    // REXSC_TUNE_PX_MIN_M (default 128): fewest output pixels for which a lane takes two of them
-    cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 128)) ? 2 : 1;
+    // Pixels per lane.  Two halve the scalar weight traffic per VALU instruction but need twice the registers
+    // (3 resident waves per SIMD instead of 5-6).  Measured on the benchmark shapes: one pixel per lane wins by
+    // 1-10 % once there are a few thousand output pixels to amortise the weights over, except for the and-or
+    // (saturation at one) instances, whose single 4-cycle instruction per weight word leaves the scalar loads
+    // exposed; few pixels (linear layers) want two.  REXSC_TUNE_PX forces 1 or 2;
+    // REXSC_TUNE_PX_MIN_M (default 128): fewest output pixels for which a lane may take two of them.
+    const bool or1_mode = !pl.wide && n_sat == 1;
+    cp.px = (!pl.wide && cp.M >= tune_env("REXSC_TUNE_PX_MIN_M", 128) && (or1_mode || cp.M < 4096)) ? 2 : 1;
+    {
+        const int forced_px = tune_env("REXSC_TUNE_PX", 0);
+        if (!pl.wide && (forced_px == 1 || (forced_px == 2 && cp.M >= 128))) cp.px = forced_px;
+    }
+    // waves resident at once: 3 per SIMD with two pixels per lane, 5 with one (register-limited)
+    const long target_waves = tune_env("REXSC_TUNE_TARGET_WAVES", cp.px == 2 ? TARGET_WAVES : 5 * 1024);
     cp.ns = n_slots >= 8 ? 4 : (n_slots >= 2 ? 2 : 1);
     {
         const int forced_ns = tune_env("REXSC_TUNE_NS", 0); // 1, 2 or 4 waves per block (tuning only)
@@ -220,7 +232,7 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
         const double overhead = tune_env("REXSC_TUNE_WAVE_OVERHEAD", 1500);
         double best = 0;
         for (int s = 1; s <= max_splits && s <= 16; s *= 2) {
-            const double rounds = (double)((waves * s + TARGET_WAVES - 1) / TARGET_WAVES);
+            const double rounds = (double)((waves * s + target_waves - 1) / target_waves);
             double cost = rounds * (work1 / s + overhead);
             if (s > 1) {
                 // the finalize pass: launch (~8 us) + partial and output bytes at ~3 TB/s, converted to the
