@@ -291,7 +291,10 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                     for (int o = 0; o < OT; o++)
                         acc[px][o] = pk_add_u16(acc[px][o], min_one(cp[px][o]) | (min_one(cn[px][o]) << 16));
             } else if (!WIDE) {
-                if (p.mode == 0) {
+                // Only the linear op (a 1x1 problem) ever asks for the "count >= n" rule.  The empty asm keeps the
+                // compiler from evaluating both rules and selecting (it did: two v_pk_min and a v_pk_sub per
+                // output and slot on the common path).
+                if (KW != 1 || p.mode == 0) {
 #pragma unroll
                     for (int px = 0; px < PX; px++)
 #pragma unroll
@@ -300,6 +303,7 @@ __global__ __launch_bounds__(64 * MAX_NS) void sc_compute_kernel(const uint32_t 
                             acc[px][o] = pk_add_u16(acc[px][o], pk_min_u16(c, p.nn));
                         }
                 } else { // [count >= n] = min(count, n) - min(count, n-1)
+                    asm volatile("" ::: "memory");
 #pragma unroll
                     for (int px = 0; px < PX; px++)
 #pragma unroll
