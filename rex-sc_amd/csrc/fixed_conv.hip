@@ -611,16 +611,34 @@ __global__ __launch_bounds__(256) void fixed_pack_w_tiles(const float *__restric
 
 constexpr int FUSED_W_ENTRIES = 2 * 9 * 2 * 64; // 16-byte entries of one (otile, pair): 36 KB
 
+// Parity term of packed int8 weights: per byte, 0 for an even weight, +1 / -1 for an odd positive / negative one.
+__device__ __forceinline__ v4i weight_parities(v4i a)
+{
+    v4i r;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t w = (uint32_t)a[i];
+        const uint32_t odd = w & 0x01010101u;         // 1 per odd byte
+        const uint32_t neg_odd = (w >> 7) & odd;      // 1 per odd negative byte
+        r[i] = (int)(((neg_odd << 8) - neg_odd) | odd); // 0xFF per odd negative byte, 0x01 per odd positive one
+    }
+    return r;
+}
+
 // PBW: 32-pixel blocks per wave; AR: rounds of 256 (padded pixel, half) entries that cover the tile.
 // A block walks over its items (blockIdx.x, + gridDim.x, ...) and their pairs as one sequence of steps; the global
 // loads of step s + 1 are issued before the MFMAs of step s and land in registers while those run.
-template <int PBW, int AR>
-__global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__restrict__ x, const int8_t *__restrict__ wpk,
+// WS (weight-stationary; every weight of the layer fits 36 KB of int8, one output-channel tile): the block quantises
+// the float32 weights itself once, keeps the int8 values of all pairs in LDS for all its items and derives the
+// parities in registers -- no weight traffic per step and no separate weight-tiling launch; wpk is then the float32
+// weight tensor [O][C][3][3].
+template <int PBW, int AR, bool WS>
+__global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__restrict__ x, const void *__restrict__ wpk,
                                                           int32_t *__restrict__ out, FusedParams p)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t s_raw[];
-    v4i *s_w = reinterpret_cast<v4i *>(s_raw);       // [h][tap][val/par][o 0..63]
-    v4i *s_a = s_w + FUSED_W_ENTRIES;                // [h][padded pixel of the tile]
+    v4i *s_w = reinterpret_cast<v4i *>(s_raw);       // [h][tap][val/par][o 0..63]; WS: [pair][h][tap][o 0..63], values only
+    v4i *s_a = s_w + (WS ? p.pairs * (FUSED_W_ENTRIES / 2) : FUSED_W_ENTRIES); // [h][padded pixel of the tile]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 31, h = lane >> 5;
@@ -660,6 +678,44 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         abase[pb] = i < p.NI ? (i * RP + r) * Wp + l_col[pb] : 0;
     }
 
+    if (WS) {
+        // All weights of the layer, once per block: a work item is four consecutive channels of one output channel
+        // (36 contiguous floats); it yields one dword (bytes = the four channels) of the nine taps' LDS entries.
+        const float *wf = reinterpret_cast<const float *>(wpk);
+        const float hi = p.P2 - 1.f;
+        uint32_t *s_wd = reinterpret_cast<uint32_t *>(s_w);
+        const int n_quads = 64 * p.pairs * 8;
+        for (int qd = threadIdx.x; qd < n_quads; qd += 256) {
+            const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
+            const int pr = rest % p.pairs, o = rest / p.pairs;
+            const int c0 = pr * 32 + hh * 16 + b * 4;
+            float v[36];
+            if (o < p.O && c0 + 4 <= p.C) { // the host has checked C % 4 == 0 and the tensor's alignment
+                const float4 *src = reinterpret_cast<const float4 *>(wf + ((long)o * p.C + c0) * 9);
+#pragma unroll
+                for (int e = 0; e < 9; e++) {
+                    const float4 f = src[e];
+                    v[4 * e] = f.x; v[4 * e + 1] = f.y; v[4 * e + 2] = f.z; v[4 * e + 3] = f.w;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 36; e++) v[e] = 0.f;
+            }
+            uint32_t *dst = s_wd + ((long)((pr * 2 + hh) * 9) * 64 + o) * 4 + b;
+#pragma unroll
+            for (int tap = 0; tap < 9; tap++) {
+                uint32_t d = 0;
+#pragma unroll
+                for (int k = 0; k < 4; k++) { // round(clamp(w * P2, 1 - P2, P2 - 1)), half to even: positive part minus negative part
+                    const int q = (int)rintf(fminf(fmaxf(v[k * 9 + tap] * p.P2, -hi), hi));
+                    d |= ((uint32_t)q & 0xffu) << (8 * k);
+                }
+                dst[tap * 64 * 4] = d;
+            }
+        }
+        __syncthreads();
+    }
+
     v16i acc[2][PBW];
 #pragma unroll
     for (int a = 0; a < 2; a++)
@@ -668,7 +724,7 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
     const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-    constexpr int WR = FUSED_W_ENTRIES / 256;
+    constexpr int WR = WS ? 1 : FUSED_W_ENTRIES / 256;
     v4i wreg[WR];
     float freg[AR][16];
 
@@ -676,9 +732,11 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         const int otile = item % p.o_tiles, tile = item / p.o_tiles;
         const int ty = tile % p.tiles_y, tg = tile / p.tiles_y;
         const int n0 = tg * p.NI, y0 = ty * p.TH;
-        const v4i *src = reinterpret_cast<const v4i *>(wpk) + ((long)otile * p.pairs + pair) * FUSED_W_ENTRIES + threadIdx.x;
+        if (!WS) {
+            const v4i *src = reinterpret_cast<const v4i *>(wpk) + ((long)otile * p.pairs + pair) * FUSED_W_ENTRIES + threadIdx.x;
 #pragma unroll
-        for (int e = 0; e < WR; e++) wreg[e] = src[e * 256];
+            for (int e = 0; e < WR; e++) wreg[e] = src[e * 256];
+        }
         // (for the first tile this base lies one row and one element before the tensor; those entries are never loaded)
         const char *xb = reinterpret_cast<const char *>(x) + (((long)n0 * p.C + pair * 32) * plane + (long)(y0 - 1) * p.W - 1) * 4;
 #pragma unroll
@@ -743,8 +801,10 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
     while (true) {
         // operands of this step: registers -> LDS (activations rounded half to even and clamped to [0, P2 - 1] on the way:
         // v_cvt_pk_u8_f32 rounds to nearest even, clamps below at zero and drops the byte into place)
+        if (!WS) {
 #pragma unroll
-        for (int e = 0; e < WR; e++) s_w[threadIdx.x + e * 256] = wreg[e];
+            for (int e = 0; e < WR; e++) s_w[threadIdx.x + e * 256] = wreg[e];
+        }
 #pragma unroll
         for (int a = 0; a < AR; a++) {
             uint32_t wds[4] = {0, 0, 0, 0};
@@ -763,14 +823,15 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         const bool more = nitem < p.n_items;
         if (more) issue(nitem, npair);
 
-        const v4i *sw = s_w + h * (9 * 2 * 64) + j;
+        const v4i *sw = WS ? s_w + (pair * 2 + h) * (9 * 64) + j : s_w + h * (9 * 2 * 64) + j;
         const v4i *sa = s_a + h * NPP;
 #pragma unroll
         for (int ky = 0; ky < 3; ky++)
 #pragma unroll
             for (int kx = 0; kx < 3; kx++) {
-                const v4i *wt = sw + (ky * 3 + kx) * 2 * 64;
-                const v4i a0 = wt[0], a1 = wt[32], q0 = wt[64], q1 = wt[96];
+                const v4i *wt = sw + (ky * 3 + kx) * (WS ? 64 : 2 * 64);
+                const v4i a0 = wt[0], a1 = wt[32];
+                const v4i q0 = WS ? weight_parities(a0) : wt[64], q1 = WS ? weight_parities(a1) : wt[96];
 #pragma unroll
                 for (int pb = 0; pb < PBW; pb++) {
                     const v4i b = sa[abase[pb] + ky * Wp + kx];
@@ -940,7 +1001,20 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         // long to hide their load latency, and the two-pass path stays ahead.  REXSC_TUNE_FIXED_FUSED: 0 never, 2 wherever it can.
         const int fused_mode = tune_flag("REXSC_TUNE_FIXED_FUSED", 1);
         if (fused_mode && fused_plan(p, q.O_pad, fp) && (fused_mode == 2 || p.H * p.W >= 512)) {
-            {
+            const int NPP = fp.NI * (fp.TH + 2) * (fp.W + 2);
+            const int PBT = ceil_div(fp.NI * fp.TH * fp.W, 32);
+            const int AR = ceil_div(2 * NPP, 256);
+            // weight-stationary: every weight of the layer as int8 in 36 KB of LDS, read as aligned float4 runs
+            const bool ws = fp.o_tiles == 1 && fp.pairs <= 2 && p.C % 4 == 0 && ((uintptr_t)w % 16) == 0 &&
+                            tune_flag("REXSC_TUNE_FIXED_WS", 1);
+            // persistent blocks: two per CU stay resident (three measured a third slower: more blocks contending for the
+            // same HBM time), then fewer until every block has the same number of items
+            const int resident = 256 * 2;
+            const int per_block = ceil_div(fp.n_items, resident);
+            unsigned grid = (unsigned)ceil_div(fp.n_items, per_block);
+            if (grid > 8 && grid % 8) grid += 8 - grid % 8;                  // XCD-aware item order needs a multiple of 8
+            if (grid > (unsigned)fp.n_items) grid = (unsigned)fp.n_items;
+            if (!ws) {
                 ProfScope prof("fixed_pack_weights", 4.0 * p.O * p.C * 9 + 32.0 * q.O_pad * q.CB * 9, stream);
                 const long entries = (long)q.O_pad * q.CB * 9;
                 hipLaunchKernelGGL(fixed_pack_w_tiles, dim3((unsigned)gridf(entries)), dim3(256), 0, stream, w, wq16, p.O, p.C,
@@ -948,13 +1022,12 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
                 REXSC_CHECK_HIP(hipGetLastError());
             }
             ProfScope prof("fixed_conv_fused", io_bytes, stream);
-            const int NPP = fp.NI * (fp.TH + 2) * (fp.W + 2);
-            const size_t lds = (size_t)(FUSED_W_ENTRIES + 2 * NPP) * 16;
-            const int PBT = ceil_div(fp.NI * fp.TH * fp.W, 32);
-            const int AR = ceil_div(2 * NPP, 256);
-            unsigned grid = (unsigned)(fp.n_items < 512 ? fp.n_items : 512); // two blocks per CU stay resident
-            if (grid > 8) grid -= grid % 8;                                   // XCD-aware item order needs a multiple of 8
-#define REXSC_FUSED(PBW_, AR_) hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_>), dim3(grid), dim3(256), lds, stream, x, wq16, out, fp)
+            const size_t lds = (size_t)((ws ? fp.pairs * (FUSED_W_ENTRIES / 2) : FUSED_W_ENTRIES) + 2 * NPP) * 16;
+#define REXSC_FUSED(PBW_, AR_)                                                                                                      \
+    do {                                                                                                                            \
+        if (ws) hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_, true>), dim3(grid), dim3(256), lds, stream, x, (const void *)w, out, fp); \
+        else hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_, false>), dim3(grid), dim3(256), lds, stream, x, (const void *)wq16, out, fp); \
+    } while (0)
             if (PBT <= 4) { if (AR <= 2) REXSC_FUSED(1, 2); else REXSC_FUSED(1, 3); }
             else { if (AR <= 2) REXSC_FUSED(2, 2); else REXSC_FUSED(2, 3); }
 #undef REXSC_FUSED

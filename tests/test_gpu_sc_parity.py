@@ -245,19 +245,24 @@ FUSED_FIXED = [
     (7, 96, 14, 14, 192),   # one image per tile, three output tiles
     (70, 8, 5, 9, 8),       # small planes, one image per tile
     (600, 8, 5, 9, 8),      # small planes, two images per tile
+    (2, 12, 20, 20, 5),     # few channels, few outputs: all weights stay in LDS, channel tail inside a half
+    (2, 64, 24, 24, 64),    # exactly one output tile and two channel pairs
 ]
 
 
-@pytest.mark.parametrize("path", ["planner", "single_pass", "two_pass"])
+@pytest.mark.parametrize("path", ["planner", "single_pass", "single_pass_tiled_weights", "two_pass"])
 @pytest.mark.parametrize("cfg", FUSED_FIXED, ids=lambda c: "_".join(str(v) for v in c))
 def test_fixed_fused_shapes_and_out_of_range_operands(cfg, path, monkeypatch):
     """Activations below zero, above one, at rounding ties and near-ties; weights likewise.  Once with the
-    library's own choice between the single-pass and the two-pass MFMA path, once with each forced."""
+    library's own choice between the single-pass and the two-pass MFMA path, once with each forced (the single
+    pass also without its weights-in-LDS variant)."""
     import fixed_extension_cuda
     N, C, H, W, O = cfg
     print("fixed fused", cfg, path, flush=True)
     if path != "planner":
-        monkeypatch.setenv("REXSC_TUNE_FIXED_FUSED", "2" if path == "single_pass" else "0")
+        monkeypatch.setenv("REXSC_TUNE_FIXED_FUSED", "0" if path == "two_pass" else "2")
+    if path == "single_pass_tiled_weights":   # never the variant that keeps all weights in LDS
+        monkeypatch.setenv("REXSC_TUNE_FIXED_WS", "0")
     rng = np.random.default_rng(sum(cfg))
     x = (rng.integers(-8, 80, size=(N, C, H, W)) / 64).astype(np.float32)            # [-1/8, 5/4) on the half grid
     x += (rng.integers(-1, 2, size=x.shape) * 2.0 ** -20).astype(np.float32)         # just below / at / above
