@@ -632,7 +632,11 @@ __device__ __forceinline__ v4i weight_parities(v4i a)
 // the float32 weights itself once, keeps the int8 values of all pairs in LDS for all its items and derives the
 // parities in registers -- no weight traffic per step and no separate weight-tiling launch; wpk is then the float32
 // weight tensor [O][C][3][3].
-template <int PBW, int AR, bool WS>
+// V4 (rows of a multiple of four pixels, 16-byte aligned tensor): a thread's entry is four neighbouring pixels of
+// one row and 16-channel half, read as sixteen 16-byte loads (one per channel) instead of four times sixteen 4-byte
+// loads -- vector-memory instruction issue, not bytes, was what the load phase of a step spent its time on.  The
+// halo columns are then never loaded: they are zeroed once.
+template <int PBW, int AR, bool WS, bool V4>
 __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__restrict__ x, const void *__restrict__ wpk,
                                                           int32_t *__restrict__ out, FusedParams p)
 {
@@ -654,6 +658,21 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
     int e_img[AR], e_row[AR];
     uint32_t e_off[AR];
     bool e_colok[AR];
+    // V4: one entry per thread = (half, image, padded row, group of four pixels); GW groups per row
+    const int GW = p.W / 4, NQ = p.NI * RP * GW;
+    int q_img = 1 << 28, q_row = 0, q_half = 0, q_lds = 0;
+    uint32_t q_off = 0;
+    if (V4 && (int)threadIdx.x < 2 * NQ) {
+        const int e = threadIdx.x;
+        q_half = e >= NQ ? 1 : 0;
+        const int pp = e - q_half * NQ;
+        const int i = pp / (RP * GW), rem = pp - i * (RP * GW);
+        q_row = rem / GW;
+        const int g = rem - q_row * GW;
+        q_img = i;
+        q_off = (uint32_t)((((long)i * p.C + q_half * 16) * plane + (long)q_row * p.W + 4 * g) * 4);
+        q_lds = q_half * NPP + (i * RP + q_row) * Wp + 4 * g + 1;
+    }
 #pragma unroll
     for (int a = 0; a < AR; a++) {
         const int e = a * 256 + threadIdx.x;
@@ -684,22 +703,33 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         const float *wf = reinterpret_cast<const float *>(wpk);
         const float hi = p.P2 - 1.f;
         uint32_t *s_wd = reinterpret_cast<uint32_t *>(s_w);
-        const int n_quads = 64 * p.pairs * 8;
-        for (int qd = threadIdx.x; qd < n_quads; qd += 256) {
+        const int n_quads = 64 * p.pairs * 8; // at most 1024: four work items per thread, all loads issued before the first use
+        float4 v4[4][9];
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int qd = it * 256 + threadIdx.x;
             const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
             const int pr = rest % p.pairs, o = rest / p.pairs;
             const int c0 = pr * 32 + hh * 16 + b * 4;
-            float v[36];
-            if (o < p.O && c0 + 4 <= p.C) { // the host has checked C % 4 == 0 and the tensor's alignment
+            if (qd < n_quads && o < p.O && c0 + 4 <= p.C) { // the host has checked C % 4 == 0 and the tensor's alignment
                 const float4 *src = reinterpret_cast<const float4 *>(wf + ((long)o * p.C + c0) * 9);
 #pragma unroll
-                for (int e = 0; e < 9; e++) {
-                    const float4 f = src[e];
-                    v[4 * e] = f.x; v[4 * e + 1] = f.y; v[4 * e + 2] = f.z; v[4 * e + 3] = f.w;
-                }
+                for (int e = 0; e < 9; e++) v4[it][e] = src[e];
             } else {
 #pragma unroll
-                for (int e = 0; e < 36; e++) v[e] = 0.f;
+                for (int e = 0; e < 9; e++) v4[it][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int qd = it * 256 + threadIdx.x;
+            if (qd >= n_quads) break;
+            const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
+            const int pr = rest % p.pairs, o = rest / p.pairs;
+            float v[36];
+#pragma unroll
+            for (int e = 0; e < 9; e++) {
+                v[4 * e] = v4[it][e].x; v[4 * e + 1] = v4[it][e].y; v[4 * e + 2] = v4[it][e].z; v[4 * e + 3] = v4[it][e].w;
             }
             uint32_t *dst = s_wd + ((long)((pr * 2 + hh) * 9) * 64 + o) * 4 + b;
 #pragma unroll
@@ -715,6 +745,13 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         }
         __syncthreads();
     }
+    if (V4) { // the halo columns of every padded row stay zero for the whole launch
+        for (int e = threadIdx.x; e < 2 * p.NI * RP * 2; e += 256) {
+            const int side = e & 1, rowi = e >> 1; // rowi counts (half, image, row)
+            const int hh = rowi / (p.NI * RP), ir = rowi - hh * (p.NI * RP);
+            s_a[hh * NPP + ir * Wp + (side ? Wp - 1 : 0)] = (v4i){0, 0, 0, 0};
+        }
+    }
 
     v16i acc[2][PBW];
 #pragma unroll
@@ -726,7 +763,8 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
     const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
     constexpr int WR = WS ? 1 : FUSED_W_ENTRIES / 256;
     v4i wreg[WR];
-    float freg[AR][16];
+    float freg[V4 ? 1 : AR][16];
+    float4 qreg[V4 ? 16 : 1];
 
     auto issue = [&](int item, int pair) {
         const int otile = item % p.o_tiles, tile = item / p.o_tiles;
@@ -736,6 +774,25 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
             const v4i *src = reinterpret_cast<const v4i *>(wpk) + ((long)otile * p.pairs + pair) * FUSED_W_ENTRIES + threadIdx.x;
 #pragma unroll
             for (int e = 0; e < WR; e++) wreg[e] = src[e * 256];
+        }
+        if (V4) {
+            // (for the first tile this base lies one row before the tensor; those rows are never loaded)
+            const char *xq = reinterpret_cast<const char *>(x) + (((long)n0 * p.C + pair * 32) * plane + (long)(y0 - 1) * p.W) * 4;
+            const int n = n0 + q_img, y = y0 + q_row - 1;
+            const bool inb = n < p.N && y >= 0 && y < p.H;
+            const int kmax = inb ? p.C - pair * 32 - q_half * 16 : 0;
+            if (kmax >= 16) {
+#pragma unroll
+                for (int k = 0; k < 16; k++) qreg[k] = *reinterpret_cast<const float4 *>(xq + k * plane * 4 + q_off);
+            } else if (kmax > 0) {
+#pragma unroll
+                for (int k = 0; k < 16; k++)
+                    qreg[k] = k < kmax ? *reinterpret_cast<const float4 *>(xq + k * plane * 4 + q_off) : make_float4(0.f, 0.f, 0.f, 0.f);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 16; k++) qreg[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            return;
         }
         // (for the first tile this base lies one row and one element before the tensor; those entries are never loaded)
         const char *xb = reinterpret_cast<const char *>(x) + (((long)n0 * p.C + pair * 32) * plane + (long)(y0 - 1) * p.W - 1) * 4;
@@ -805,13 +862,28 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
 #pragma unroll
             for (int e = 0; e < WR; e++) s_w[threadIdx.x + e * 256] = wreg[e];
         }
+        if (V4) {
+            if ((int)threadIdx.x < 2 * NQ) {
 #pragma unroll
-        for (int a = 0; a < AR; a++) {
-            uint32_t wds[4] = {0, 0, 0, 0};
+                for (int px = 0; px < 4; px++) {
+                    uint32_t wds[4] = {0, 0, 0, 0};
 #pragma unroll
-            for (int k = 0; k < 16; k++)
-                wds[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(fminf(freg[a][k] * p.P2, top), k & 3, wds[k >> 2]);
-            if (a * 256 + (int)threadIdx.x < 2 * NPP) s_a[a * 256 + threadIdx.x] = (v4i){(int)wds[0], (int)wds[1], (int)wds[2], (int)wds[3]};
+                    for (int k = 0; k < 16; k++) {
+                        const float f = px == 0 ? qreg[k].x : px == 1 ? qreg[k].y : px == 2 ? qreg[k].z : qreg[k].w;
+                        wds[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(fminf(f * p.P2, top), k & 3, wds[k >> 2]);
+                    }
+                    s_a[q_lds + px] = (v4i){(int)wds[0], (int)wds[1], (int)wds[2], (int)wds[3]};
+                }
+            }
+        } else {
+#pragma unroll
+            for (int a = 0; a < AR; a++) {
+                uint32_t wds[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int k = 0; k < 16; k++)
+                    wds[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(fminf(freg[a][k] * p.P2, top), k & 3, wds[k >> 2]);
+                if (a * 256 + (int)threadIdx.x < 2 * NPP) s_a[a * 256 + threadIdx.x] = (v4i){(int)wds[0], (int)wds[1], (int)wds[2], (int)wds[3]};
+            }
         }
         __syncthreads();
         // results of the item that ended with the previous step: stored here, before the next loads are issued, so
@@ -1023,13 +1095,19 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
             }
             ProfScope prof("fixed_conv_fused", io_bytes, stream);
             const size_t lds = (size_t)((ws ? fp.pairs * (FUSED_W_ENTRIES / 2) : FUSED_W_ENTRIES) + 2 * NPP) * 16;
-#define REXSC_FUSED(PBW_, AR_)                                                                                                      \
+            // float4 loads along the rows: rows of a multiple of four pixels, 16-byte aligned tensor
+            const bool v4 = p.W % 4 == 0 && ((uintptr_t)x % 16) == 0 && 2 * fp.NI * (fp.TH + 2) * (p.W / 4) <= 256 &&
+                            tune_flag("REXSC_TUNE_FIXED_V4", 1);
+#define REXSC_FUSED2(PBW_, AR_, V4_)                                                                                                \
     do {                                                                                                                            \
-        if (ws) hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_, true>), dim3(grid), dim3(256), lds, stream, x, (const void *)w, out, fp); \
-        else hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_, false>), dim3(grid), dim3(256), lds, stream, x, (const void *)wq16, out, fp); \
+        if (ws) hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_, true, V4_>), dim3(grid), dim3(256), lds, stream, x, (const void *)w, out, fp); \
+        else hipLaunchKernelGGL((fixed_fused_kernel<PBW_, AR_, false, V4_>), dim3(grid), dim3(256), lds, stream, x, (const void *)wq16, out, fp); \
     } while (0)
-            if (PBT <= 4) { if (AR <= 2) REXSC_FUSED(1, 2); else REXSC_FUSED(1, 3); }
+#define REXSC_FUSED(PBW_, AR_) REXSC_FUSED2(PBW_, AR_, false)
+            if (v4) { if (PBT <= 4) REXSC_FUSED2(1, 1, true); else REXSC_FUSED2(2, 1, true); }
+            else if (PBT <= 4) { if (AR <= 2) REXSC_FUSED(1, 2); else REXSC_FUSED(1, 3); }
             else { if (AR <= 2) REXSC_FUSED(2, 2); else REXSC_FUSED(2, 3); }
+#undef REXSC_FUSED2
 #undef REXSC_FUSED
             REXSC_CHECK_HIP(hipGetLastError());
             return REXSC_OK;

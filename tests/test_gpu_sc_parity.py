@@ -247,6 +247,9 @@ FUSED_FIXED = [
     (600, 8, 5, 9, 8),      # small planes, two images per tile
     (2, 12, 20, 20, 5),     # few channels, few outputs: all weights stay in LDS, channel tail inside a half
     (2, 64, 24, 24, 64),    # exactly one output tile and two channel pairs
+    (3, 40, 12, 36, 70),    # rows of a multiple of four pixels (16-byte loads), ragged row tiles, two output tiles
+    (2, 33, 10, 16, 64),    # 16-byte loads with a channel tail of one
+    (600, 8, 4, 8, 8),      # small planes of a multiple of four pixels per row: two images per tile with 16-byte loads
 ]
 
 
