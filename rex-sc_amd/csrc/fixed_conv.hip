@@ -697,62 +697,6 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
         abase[pb] = i < p.NI ? (i * RP + r) * Wp + l_col[pb] : 0;
     }
 
-    if (WS) {
-        // All weights of the layer, once per block: a work item is four consecutive channels of one output channel
-        // (36 contiguous floats); it yields one dword (bytes = the four channels) of the nine taps' LDS entries.
-        const float *wf = reinterpret_cast<const float *>(wpk);
-        const float hi = p.P2 - 1.f;
-        uint32_t *s_wd = reinterpret_cast<uint32_t *>(s_w);
-        const int n_quads = 64 * p.pairs * 8; // at most 1024: four work items per thread, all loads issued before the first use
-        float4 v4[4][9];
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int qd = it * 256 + threadIdx.x;
-            const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
-            const int pr = rest % p.pairs, o = rest / p.pairs;
-            const int c0 = pr * 32 + hh * 16 + b * 4;
-            if (qd < n_quads && o < p.O && c0 + 4 <= p.C) { // the host has checked C % 4 == 0 and the tensor's alignment
-                const float4 *src = reinterpret_cast<const float4 *>(wf + ((long)o * p.C + c0) * 9);
-#pragma unroll
-                for (int e = 0; e < 9; e++) v4[it][e] = src[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 9; e++) v4[it][e] = make_float4(0.f, 0.f, 0.f, 0.f);
-            }
-        }
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            const int qd = it * 256 + threadIdx.x;
-            if (qd >= n_quads) break;
-            const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
-            const int pr = rest % p.pairs, o = rest / p.pairs;
-            float v[36];
-#pragma unroll
-            for (int e = 0; e < 9; e++) {
-                v[4 * e] = v4[it][e].x; v[4 * e + 1] = v4[it][e].y; v[4 * e + 2] = v4[it][e].z; v[4 * e + 3] = v4[it][e].w;
-            }
-            uint32_t *dst = s_wd + ((long)((pr * 2 + hh) * 9) * 64 + o) * 4 + b;
-#pragma unroll
-            for (int tap = 0; tap < 9; tap++) {
-                uint32_t d = 0;
-#pragma unroll
-                for (int k = 0; k < 4; k++) { // round(clamp(w * P2, 1 - P2, P2 - 1)), half to even: positive part minus negative part
-                    const int q = (int)rintf(fminf(fmaxf(v[k * 9 + tap] * p.P2, -hi), hi));
-                    d |= ((uint32_t)q & 0xffu) << (8 * k);
-                }
-                dst[tap * 64 * 4] = d;
-            }
-        }
-        __syncthreads();
-    }
-    if (V4) { // the halo columns of every padded row stay zero for the whole launch
-        for (int e = threadIdx.x; e < 2 * p.NI * RP * 2; e += 256) {
-            const int side = e & 1, rowi = e >> 1; // rowi counts (half, image, row)
-            const int hh = rowi / (p.NI * RP), ir = rowi - hh * (p.NI * RP);
-            s_a[hh * NPP + ir * Wp + (side ? Wp - 1 : 0)] = (v4i){0, 0, 0, 0};
-        }
-    }
-
     v16i acc[2][PBW];
 #pragma unroll
     for (int a = 0; a < 2; a++)
@@ -853,7 +797,72 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
     const int G = gridDim.x;
     const int first = (G % 8 == 0) ? (int)(blockIdx.x % 8) * (G / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
     int item = first, pair = 0, pending = -1;
-    issue(item, pair);
+    issue(item, pair); // the first activations are on their way while the weights are being prepared
+    if (WS) {
+        // All weights of the layer, once per block: a work item is four consecutive channels of one output channel
+        // (36 contiguous floats); it yields one dword (bytes = the four channels) of the nine taps' LDS entries.
+        const float *wf = reinterpret_cast<const float *>(wpk);
+        const float hi = p.P2 - 1.f;
+        uint32_t *s_wd = reinterpret_cast<uint32_t *>(s_w);
+        const int n_quads = 64 * p.pairs * 8; // at most 1024: four work items per thread
+        for (int it0 = 0; it0 < 4; it0 += 2) { // two batches of two work items: their loads are in flight together
+        float4 v4[2][9];
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int qd = (it0 + it) * 256 + threadIdx.x;
+            const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
+            const int pr = rest % p.pairs, o = rest / p.pairs;
+            const int c0 = pr * 32 + hh * 16 + b * 4;
+            if (qd < n_quads && o < p.O && c0 + 4 <= p.C) { // the host has checked C % 4 == 0 and the tensor's alignment
+                const float4 *src = reinterpret_cast<const float4 *>(wf + ((long)o * p.C + c0) * 9);
+#pragma unroll
+                for (int e = 0; e < 9; e++) v4[it][e] = src[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 9; e++) v4[it][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int qd = (it0 + it) * 256 + threadIdx.x;
+            if (qd >= n_quads) break;
+            const int b = qd & 3, hh = (qd >> 2) & 1, rest = qd >> 3;
+            const int pr = rest % p.pairs, o = rest / p.pairs;
+            float v[36];
+#pragma unroll
+            for (int e = 0; e < 9; e++) {
+                v[4 * e] = v4[it][e].x; v[4 * e + 1] = v4[it][e].y; v[4 * e + 2] = v4[it][e].z; v[4 * e + 3] = v4[it][e].w;
+            }
+            uint32_t *dst = s_wd + ((long)((pr * 2 + hh) * 9) * 64 + o) * 4 + b;
+            // round(clamp(w * P2, 1 - P2, P2 - 1)), half to even (positive part minus negative part), as two instructions
+            // per weight: w * P2 + 1.5 * 2^23 in one fma leaves the rounded integer in the low mantissa bits (two's
+            // complement, exact for |w * P2| < 2^22), and clamping there equals clamping before the rounding because
+            // the bounds are integers.  Larger magnitudes and infinities end at the bounds as well; v_perm_b32 gathers
+            // the low bytes.
+            const float magic = 12582912.f;
+            uint32_t qb[36];
+#pragma unroll
+            for (int e = 0; e < 36; e++)
+                qb[e] = __float_as_uint(__builtin_amdgcn_fmed3f(fmaf(v[e], p.P2, magic), magic - hi, magic + hi));
+#pragma unroll
+            for (int tap = 0; tap < 9; tap++) {
+                // bytes 0 of the four channels' words -> one dword (selector bytes: 0..3 = second operand, 4..7 = first)
+                const uint32_t lo = __builtin_amdgcn_perm(qb[9 + tap], qb[tap], 0x0c0c0400u);       // [k0, k1, 0, 0]
+                const uint32_t hi2 = __builtin_amdgcn_perm(qb[27 + tap], qb[18 + tap], 0x04000c0cu); // [0, 0, k2, k3]
+                dst[tap * 64 * 4] = lo | hi2;
+            }
+        }
+        }
+        // (no barrier here: the one behind the first step's LDS writes orders these writes before any MFMA as well)
+    }
+    if (V4) { // the halo columns of every padded row stay zero for the whole launch
+        for (int e = threadIdx.x; e < 2 * p.NI * RP * 2; e += 256) {
+            const int side = e & 1, rowi = e >> 1; // rowi counts (half, image, row)
+            const int hh = rowi / (p.NI * RP), ir = rowi - hh * (p.NI * RP);
+            s_a[hh * NPP + ir * Wp + (side ? Wp - 1 : 0)] = (v4i){0, 0, 0, 0};
+        }
+    }
+
     const float top = p.P2 - 1.f;
     while (true) {
         // operands of this step: registers -> LDS (activations rounded half to even and clamped to [0, P2 - 1] on the way:
