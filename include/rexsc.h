@@ -32,6 +32,12 @@ enum {
 };
 
 const char *rexsc_last_error(void);
+
+/* ABI version of the library.  It changes whenever a descriptor below changes its layout or an entry point its
+ * signature; a caller built against another header must refuse to go on.  Every descriptor also starts with its own
+ * size in bytes (struct_size = sizeof of the structure as the caller's header declares it): the library rejects a
+ * descriptor whose size is not the one it was compiled with instead of reading past it. */
+#define REXSC_ABI_VERSION 200
 int rexsc_version(void);
 
 /* One-time per-device set-up (LFSR sequence tables).  Called implicitly by the ops; exposed
@@ -48,6 +54,7 @@ int rexsc_init(rexsc_stream_t stream);
  * desc.xnor = 1 switches the stream generators to those of the reference's CUDA kernels.
  */
 typedef struct rexsc_conv_desc {
+    int32_t struct_size;         /* sizeof(rexsc_conv_desc) */
     int32_t N, C, H, W;          /* activation dims, UNPADDED */
     int32_t O, KH, KW;           /* weight dims [O][C][KH][KW] */
     int32_t pad_h, pad_w;        /* zero padding of axis 2 / axis 3 (the reference's padding[1] / padding[0]) */
@@ -89,9 +96,20 @@ int rexsc_conv2d_orn(const rexsc_conv_desc *d, const float *x, const float *w,
  *    and "pos - neg" passes of :1181-1182, 1273-1274, 1317 done in the kernel that produces the sums (any of the
  *    three int16 outputs may then be NULL and is not written);
  *  - weight_streams: a caller-owned buffer of rexsc_conv2d_weight_streams_bytes() that receives the weight
- *    bitstreams (and the generator table that goes with the descriptor).  With weight_streams_valid != 0 it
- *    already holds them -- same descriptor, same weights -- and generation is skipped (w may then be NULL):
- *    frozen weights (evaluation, utils_class.py:54 under no_grad) are expanded once, not per call. */
+ *    bitstreams, the generator table that goes with the descriptor and a copy of the weights they were made
+ *    from: frozen weights (evaluation, utils_class.py:54 under no_grad) are expanded once, not per call.
+ *    weight_streams_valid says what the buffer holds when the call starts:
+ *      REXSC_WSTREAMS_FILL    nothing: generate, and keep the copy of w;
+ *      REXSC_WSTREAMS_TRUST   the streams of this descriptor and of these weight values, on the caller's word:
+ *                             generation is skipped and w may be NULL;
+ *      REXSC_WSTREAMS_VERIFY  the streams of this descriptor, filled by an earlier call on the same device; whether
+ *                             the weights are still the same is decided ON THE DEVICE: a small kernel compares w
+ *                             bit for bit with the kept copy (updating it) and the generator's blocks return at
+ *                             once when nothing differs.  No host synchronisation; in-place edits of w that no
+ *                             host-side bookkeeping sees (the reference's own `p.weight.data.clamp_(-1, 0.999)`,
+ *                             utils_own.py:187-190) are caught.  Under HIP graph capture the comparison is part
+ *                             of the graph and repeats on every replay. */
+enum { REXSC_WSTREAMS_FILL = 0, REXSC_WSTREAMS_TRUST = 1, REXSC_WSTREAMS_VERIFY = 2 };
 size_t rexsc_conv2d_weight_streams_bytes(const rexsc_conv_desc *d);
 int rexsc_conv2d_orn_ex(const rexsc_conv_desc *d, const float *x, const float *w,
                         int16_t *out_pos, int16_t *out_neg, int16_t *out_diff, float *out_value,
@@ -117,9 +135,12 @@ int rexsc_conv2d_orn_noalloc(const rexsc_conv_desc *d, const float *x, const flo
  * accumulated, and bin_config < 0 selects the "count >= n_sat" rule, as in the reference.
  */
 typedef struct rexsc_linear_desc {
+    int32_t struct_size;         /* sizeof(rexsc_linear_desc) */
     int32_t B, C, O;
     int32_t bit_length, lfsr_length, gen_config, bin_config;
     int32_t total_width, load_width, load_wait;
+    int32_t act_fake_quant;      /* as in rexsc_conv_desc: k > 0 applies the layers' fake quantisation with       */
+    int32_t weight_fake_quant;   /* prec = k - 1 to the operand inside the generator (utils_class.py:196-201)    */
 } rexsc_linear_desc;
 
 size_t rexsc_linear_workspace_bytes(const rexsc_linear_desc *d);
@@ -128,9 +149,9 @@ int rexsc_linear_orn(const rexsc_linear_desc *d, const float *x, const float *w,
                      void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
 
 /* rexsc_linear_orn with the weight bitstreams in a caller-owned buffer of rexsc_linear_weight_streams_bytes(d)
- * bytes, as rexsc_conv2d_orn_ex keeps them for the conv op: weight_streams_valid != 0 promises that the buffer
- * still holds the streams a previous call with the same descriptor and the same weight values generated; the
- * weight generator is then skipped (w may be NULL).  The reference regenerates them on every call
+ * bytes, as rexsc_conv2d_orn_ex keeps them for the conv op (weight_streams_valid: REXSC_WSTREAMS_FILL / _TRUST /
+ * _VERIFY with the same meaning; the batch size B is not part of what the buffer depends on as long as
+ * rexsc_linear_weight_streams_bytes() returns the same value).  The reference regenerates them on every call
  * (sc_matmul.cpp:576-676) although its layers hold their weights fixed in evaluation (utils_class.py:54). */
 size_t rexsc_linear_weight_streams_bytes(const rexsc_linear_desc *d);
 int rexsc_linear_orn_ex(const rexsc_linear_desc *d, const float *x, const float *w,
@@ -236,6 +257,7 @@ void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint3
  * rounding adder selected by add_config (0 fixed_add, 1 fixed_add_or, >=2 pairwise OR2).
  * x float32 NCHW [N][C][H][W], w float32 [O][C][KH][KW], out int32 NCHW = pos - neg. */
 typedef struct rexsc_fixed_desc {
+    int32_t struct_size;         /* sizeof(rexsc_fixed_desc) */
     int32_t N, C, H, W, O, KH, KW;
     int32_t pad_h, pad_w, stride_h, stride_w;
     int32_t add_config, precision_in, precision_out;

@@ -9,26 +9,39 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "librexsc.so")
 NOALLOC_SCRATCH_BYTES = 32 << 20  # REXSC_NOALLOC_SCRATCH_BYTES of include/rexsc.h
+ABI_VERSION = 200                 # REXSC_ABI_VERSION of include/rexsc.h: the layout the structures below mirror
+WSTREAMS_FILL, WSTREAMS_TRUST, WSTREAMS_VERIFY = 0, 1, 2  # REXSC_WSTREAMS_*
 _lib = None
 
 
-class ConvDesc(ctypes.Structure):
+class _Desc(ctypes.Structure):
+    """A descriptor of include/rexsc.h.  Its first field is its own size, filled here: positional arguments start
+    at the field after it.  The library refuses a descriptor of any other size."""
+
+    def __init__(self, *args, **kwargs):
+        super().__init__(ctypes.sizeof(type(self)), *args, **kwargs)
+
+    def key(self):
+        return tuple(getattr(self, f[0]) for f in self._fields_)
+
+
+class ConvDesc(_Desc):
     _fields_ = [(n, ctypes.c_int32) for n in (
-        "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
+        "struct_size", "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
         "bit_length", "lfsr_length", "gen_config", "bin_config",
         "total_width", "load_width", "load_wait", "act_channels_last", "weight_channels_last", "xnor",
         "act_fake_quant", "weight_fake_quant")]
 
 
-class LinearDesc(ctypes.Structure):
+class LinearDesc(_Desc):
     _fields_ = [(n, ctypes.c_int32) for n in (
-        "B", "C", "O", "bit_length", "lfsr_length", "gen_config", "bin_config",
-        "total_width", "load_width", "load_wait")]
+        "struct_size", "B", "C", "O", "bit_length", "lfsr_length", "gen_config", "bin_config",
+        "total_width", "load_width", "load_wait", "act_fake_quant", "weight_fake_quant")]
 
 
-class FixedDesc(ctypes.Structure):
+class FixedDesc(_Desc):
     _fields_ = [(n, ctypes.c_int32) for n in (
-        "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
+        "struct_size", "N", "C", "H", "W", "O", "KH", "KW", "pad_h", "pad_w", "stride_h", "stride_w",
         "add_config", "precision_in", "precision_out")]
 
 
@@ -92,6 +105,10 @@ def lib():
                 "librexsc.so is missing (%s): build it with `python rex-sc_amd/build.py`; "
                 "there is no fallback path" % LIB_PATH)
         handle = ctypes.CDLL(LIB_PATH)
+        handle.rexsc_version.restype = ctypes.c_int
+        if handle.rexsc_version() != ABI_VERSION:
+            raise RuntimeError("librexsc.so reports ABI version %d, this binding mirrors version %d: rebuild it with "
+                               "`python rex-sc_amd/build.py --force`" % (handle.rexsc_version(), ABI_VERSION))
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype = res

@@ -87,45 +87,47 @@ def _empty_out(shape, dtype, device, channels_last):
 
 
 class WeightStreamCache:
-    """Weight bitstreams of one weight tensor, kept between calls while the weights do not change (evaluation,
-    frozen layers).  The owner -- the layer that holds the parameter -- passes it to sc_conv2d together with the
-    PARAMETER whose values the streams were generated from; an entry is reused while that tensor's storage pointer and
-    version counter are unchanged (in-place updates by an optimiser bump the counter, `.data = ...` swaps the pointer)
-    and the call's descriptor (shapes, stream length, generator, ...) is the same."""
+    """Weight bitstreams of one layer, kept between calls (evaluation, frozen layers) in buffers keyed by the call's
+    descriptor.  Whether a kept buffer still belongs to the current weight VALUES is never decided on the host: no
+    host-side stamp sees every edit (`p.data.clamp_()`, which the reference's own training loop uses,
+    utils_own.py:187-190, changes neither the storage pointer nor the tensor's version counter).  A buffer that
+    exists is handed to the library in VERIFY mode: a small kernel compares the weights bit for bit with the copy the
+    buffer holds and the generator runs on the device only if something differs -- no synchronisation, and any
+    edit of the weights, by any route, is caught.  A new buffer is handed over in FILL mode."""
 
     def __init__(self, max_entries=4):
         self.entries = {}
         self.max_entries = max_entries
-        self.hits = 0
-        self.misses = 0
+        self.hits = 0    # calls that reused a buffer (the device decided whether to regenerate)
+        self.misses = 0  # calls that had to allocate and fill one
 
-    def lookup(self, owner, desc_key, nbytes, device):
-        """-> (buffer, valid).  A fresh or stale entry comes back with valid = False and is then filled by the call."""
-        stamp = (owner.data_ptr(), owner._version, str(device))
-        ent = self.entries.get(desc_key)
-        if ent is not None and ent[0] == stamp and ent[1].numel() >= nbytes:
+    def lookup(self, desc_key, nbytes, device):
+        """-> (buffer, mode) with mode one of _lib.WSTREAMS_VERIFY (kept buffer) / _lib.WSTREAMS_FILL (new buffer)."""
+        key = (desc_key, str(device), int(nbytes), os.environ.get("REXSC_FOLD_TAPS"), os.environ.get("REXSC_SNG_MODE"))
+        buf = self.entries.get(key)
+        if buf is not None:
             self.hits += 1
-            return ent[1], True
+            return buf, _lib.WSTREAMS_VERIFY
         self.misses += 1
-        if ent is None and len(self.entries) >= self.max_entries:
+        if len(self.entries) >= self.max_entries:
             self.entries.pop(next(iter(self.entries)))
         buf = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
-        self.entries[desc_key] = (stamp, buf)
-        return buf, False
+        self.entries[key] = buf
+        return buf, _lib.WSTREAMS_FILL
 
     def clear(self):
         self.entries.clear()
 
 
 def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
-              want_split=True, want_diff=False, xnor=False, want_value=False, weight_cache=None, weight_owner=None,
+              want_split=True, want_diff=False, xnor=False, want_value=False, weight_cache=None,
               act_fake_quant=None, weight_fake_quant=None):
     """SC conv2d on the HIP path.  padding=(p0,p1): p0 pads the LAST axis, p1 axis 2, as the
     reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2.
     -> (pos, neg, diff) int16, plus the float32 tensor pos / L - neg / L as a fourth element when want_value.
-    weight_cache / weight_owner: a WeightStreamCache and the tensor whose pointer and version identify w's values
-    (default: w itself).  act_fake_quant / weight_fake_quant: precision of the layers' fake quantisation to apply to
-    the operand inside the generators (None: operand as given)."""
+    weight_cache: a WeightStreamCache that keeps w's bitstreams between calls (the device checks on every call that
+    they still belong to w's values).  act_fake_quant / weight_fake_quant: precision of the layers' fake quantisation
+    to apply to the operand inside the generators (None: operand as given)."""
     _require_cuda(x, w)
     if x.dim() != 4 or w.dim() != 4 or x.size(1) != w.size(1):
         raise RuntimeError("conv2d: expected input [N,C,H,W] and weight [O,C,KH,KW] with equal C, got %s and %s"
@@ -160,33 +162,34 @@ def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_con
             _lib.check(rc, "rexsc_conv2d_orn")
             return pos, neg, diff
         value = mk(want_value, torch.float32)
-        wbuf, valid = None, False
+        wbuf, mode = None, _lib.WSTREAMS_FILL
         if weight_cache is not None:
-            key = tuple(getattr(d, f[0]) for f in d._fields_)
-            wbuf, valid = weight_cache.lookup(w if weight_owner is None else weight_owner, key,
-                                              L.rexsc_conv2d_weight_streams_bytes(ctypes.byref(d)), x.device)
+            wbuf, mode = weight_cache.lookup(("conv",) + d.key(), L.rexsc_conv2d_weight_streams_bytes(ctypes.byref(d)),
+                                             x.device)
         rc = L.rexsc_conv2d_orn_ex(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(diff), _ptr(value),
-                                   _ptr(wbuf), wbuf.numel() if wbuf is not None else 0, int(valid),
+                                   _ptr(wbuf), wbuf.numel() if wbuf is not None else 0, mode,
                                    _ptr(ws), ws.numel(), _stream())
         _lib.check(rc, "rexsc_conv2d_orn_ex")
     return (pos, neg, diff, value) if want_value else (pos, neg, diff)
 
 
-def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config, weight_cache=None, weight_owner=None,
-              weight_transform=None):
-    """SC linear on the HIP path -> (pos, neg) int32 [B,O].  weight_cache / weight_owner: a WeightStreamCache and the
-    tensor whose pointer and version identify the weight values (default: w itself); weight_transform: applied to w
-    only when the streams have to be generated (the layer's fake quantisation), and part of what the cache entry
-    stands for -- the caller keeps it the same function for one cache."""
+def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config, weight_cache=None,
+              act_fake_quant=None, weight_fake_quant=None):
+    """SC linear on the HIP path -> (pos, neg) int32 [B,O].  weight_cache: a WeightStreamCache that keeps w's
+    bitstreams between calls (the device checks on every call that they still belong to w's values);
+    act_fake_quant / weight_fake_quant: precision of the layers' fake quantisation to apply to the operand inside
+    the generators (None: operand as given)."""
     _require_cuda(x, w)
     if x.dim() != 2 or w.dim() != 2 or x.size(1) != w.size(1):
         raise RuntimeError("linear: expected input [B,C] and weight [O,C], got %s and %s"
                            % (tuple(x.shape), tuple(w.shape)))
     xc = x.detach().float().contiguous()
+    wc = w.detach().float().contiguous()
     B, C = xc.shape
     O = w.shape[0]
+    fq = lambda p: 0 if p is None else int(p) + 1
     d = _lib.LinearDesc(B, C, O, int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
-                        int(prog_load[0]), int(prog_load[1]), int(prog_load[2]))
+                        int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), fq(act_fake_quant), fq(weight_fake_quant))
     L = _lib.lib()
     if B == 0:
         return (torch.empty((0, O), dtype=torch.int32, device=x.device),
@@ -198,23 +201,17 @@ def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config, 
         pos = torch.empty((B, O), dtype=torch.int32, device=x.device)
         neg = torch.empty((B, O), dtype=torch.int32, device=x.device)
         ws = _workspace(ws_bytes, x.device)
-        wbuf, valid = None, False
-        if weight_cache is not None:
-            # the batch size is not part of the key: the weight streams do not depend on it
-            key = ("linear", C, O, int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
-                   tuple(int(v) for v in prog_load))
-            wbuf, valid = weight_cache.lookup(weight_owner if weight_owner is not None else w, key,
-                                              L.rexsc_linear_weight_streams_bytes(ctypes.byref(d)), x.device)
-        if not valid and weight_transform is not None:
-            w = weight_transform(w)
-        wc = w.detach().float().contiguous()
-        if wbuf is None:
+        if weight_cache is None:
             rc = L.rexsc_linear_orn(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws), ws.numel(),
                                     _stream())
             _lib.check(rc, "rexsc_linear_orn")
         else:
+            # The batch size is not part of the key: the weight streams do not depend on it.  The buffer's size is:
+            # it says whether the buffer also carries the activation generator's table, which small batches go without.
+            key = ("linear",) + d.key()[2:]
+            wbuf, mode = weight_cache.lookup(key, L.rexsc_linear_weight_streams_bytes(ctypes.byref(d)), x.device)
             rc = L.rexsc_linear_orn_ex(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(wbuf), wbuf.numel(),
-                                       1 if valid else 0, _ptr(ws), ws.numel(), _stream())
+                                       mode, _ptr(ws), ws.numel(), _stream())
             _lib.check(rc, "rexsc_linear_orn_ex")
     return pos, neg
 

@@ -985,7 +985,7 @@ static bool fused_plan(const FixedParams &p, int O_pad, FusedParams &f)
 
 static int fixed_plan(const rexsc_fixed_desc *d, FixedParams &p, size_t &off_w, size_t &total)
 {
-    REXSC_CHECK_ARG(d != nullptr, "null descriptor");
+    REXSC_CHECK_DESC(d, rexsc_fixed_desc);
     REXSC_CHECK_ARG(d->N > 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->O > 0 && d->KH > 0 && d->KW > 0,
                     "non-positive dimension");
     REXSC_CHECK_ARG(d->pad_h >= 0 && d->pad_w >= 0 && d->stride_h > 0 && d->stride_w > 0, "bad padding/stride");

@@ -132,15 +132,21 @@ __global__ __launch_bounds__(256) void valu_probe_kernel(int iters, uint32_t w0,
 extern "C" int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream_, double *ms_out, double *lane_ops_out)
 {
     hipStream_t stream = (hipStream_t)stream_;
-    REXSC_CHECK_ARG(mode >= 0 && mode <= 4 && iters > 0 && ms_out && lane_ops_out, "valu probe: bad arguments");
+    // 100000 iterations of 64 slots are about 20 ms per launch: long enough for any measurement
+    REXSC_CHECK_ARG(mode >= 0 && mode <= 4 && iters > 0 && iters <= 100000 && ms_out && lane_ops_out,
+                    "valu probe: mode 0..4, 1 <= iters <= 100000");
     hipDeviceProp_t prop;
     int dev = 0;
     REXSC_CHECK_HIP(hipGetDevice(&dev));
     REXSC_CHECK_HIP(hipGetDeviceProperties(&prop, dev));
     const int blocks = prop.multiProcessorCount * 8; // 4 waves per block: 8 waves per SIMD
-    hipEvent_t e0, e1;
-    REXSC_CHECK_HIP(hipEventCreate(&e0));
-    REXSC_CHECK_HIP(hipEventCreate(&e1));
+    struct Events { // destroyed on every way out
+        hipEvent_t a = nullptr, b = nullptr;
+        ~Events() { if (a) (void)hipEventDestroy(a); if (b) (void)hipEventDestroy(b); }
+    } ev;
+    REXSC_CHECK_HIP(hipEventCreate(&ev.a));
+    REXSC_CHECK_HIP(hipEventCreate(&ev.b));
+    const hipEvent_t e0 = ev.a, e1 = ev.b;
     for (int rep = 0; rep < 2; rep++) { // the first launch warms the clocks up
         REXSC_CHECK_HIP(hipEventRecord(e0, stream));
         switch (mode) {
@@ -156,8 +162,6 @@ extern "C" int rexsc_valu_probe(int mode, int iters, rexsc_stream_t stream_, dou
     }
     float ms = 0.f;
     REXSC_CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     *ms_out = ms;
     // VALU instructions per lane: 64 slots per iteration, two instructions each for the pairs, one otherwise
     *lane_ops_out = (double)blocks * 256.0 * (double)iters * 64.0 * (mode == 0 || mode == 2 ? 2.0 : 1.0);

@@ -30,6 +30,15 @@ void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
         }                                                                                  \
     } while (0)
 
+// A descriptor carries the size its caller's header gives it: anything else was built against another ABI.
+#define REXSC_CHECK_DESC(d, type)                                                                                       \
+    do {                                                                                                                \
+        REXSC_CHECK_ARG((d) != nullptr, "null descriptor");                                                             \
+        REXSC_CHECK_ARG((d)->struct_size == (int32_t)sizeof(type),                                                      \
+                        #type ": struct_size %d, this library (ABI %d) expects %zu -- caller and library were built "   \
+                        "from different headers", (int)(d)->struct_size, REXSC_ABI_VERSION, sizeof(type));             \
+    } while (0)
+
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 

@@ -3,6 +3,7 @@
 #include <stdarg.h>
 #include <stdlib.h>
 #include <string.h>
+#include <atomic>
 #include <mutex>
 
 #include "sc_compute.h"
@@ -50,6 +51,8 @@ struct ScPlan {
     size_t off_w2, off_a2, w2_bytes;                          // folded streams in the workspace
     size_t wstream_off_w2;                                    // ... and in a separate weight-stream buffer
     size_t wstream_off_tab, wstream_total; // layout of a separate weight-stream buffer: [Wst][state-plane table]
+    size_t wstream_off_snap, wstream_off_flag; // ... [folded streams][copy of the weights][change flag]
+    size_t w_elems;                            // O*C*KH*KW
     size_t tab_a_words; // state-plane table of the bit-sliced activation generator (0: ballot generator)
 };
 
@@ -276,13 +279,24 @@ int make_plan(ScPlan &pl, int N, int C, int H, int W, int O, int KH, int KW, int
         pl.wstream_off_w2 = pl.wstream_total;
         pl.wstream_total += align_up(pl.w2_bytes, WS_ALIGN);
     }
+    pl.w_elems = (size_t)O * C * KH * KW;
+    pl.wstream_off_snap = pl.wstream_total;
+    pl.wstream_off_flag = pl.wstream_off_snap + align_up(pl.w_elems * 4, WS_ALIGN);
+    pl.wstream_total = pl.wstream_off_flag + WS_ALIGN;
     cp.inv_L = 1.0f / (float)bit_length;
     return REXSC_OK;
 }
 
+// Epochs of the weight-stream change flag: one per call that fills or verifies a kept buffer, never reused.
+unsigned long long next_epoch()
+{
+    static std::atomic<unsigned long long> counter{0x5243000000000001ull};
+    return counter.fetch_add(1);
+}
+
 int plan_conv(ScPlan &pl, const rexsc_conv_desc *d)
 {
-    REXSC_CHECK_ARG(d != nullptr, "null descriptor");
+    REXSC_CHECK_DESC(d, rexsc_conv_desc);
     return make_plan(pl, d->N, d->C, d->H, d->W, d->O, d->KH, d->KW, d->pad_h, d->pad_w, d->stride_h, d->stride_w,
                      d->bit_length, d->lfsr_length, d->gen_config, d->bin_config, d->total_width, d->load_width,
                      d->load_wait, d->act_channels_last != 0, d->weight_channels_last != 0, false, d->xnor != 0,
@@ -291,10 +305,11 @@ int plan_conv(ScPlan &pl, const rexsc_conv_desc *d)
 
 int plan_linear(ScPlan &pl, const rexsc_linear_desc *d)
 {
-    REXSC_CHECK_ARG(d != nullptr, "null descriptor");
+    REXSC_CHECK_DESC(d, rexsc_linear_desc);
     // batch rows become the pixels of a single 1 x B "image" in channels-last order
     int rc = make_plan(pl, 1, d->C, 1, d->B, d->O, 1, 1, 0, 0, 1, 1, d->bit_length, d->lfsr_length, d->gen_config,
-                       d->bin_config, d->total_width, d->load_width, d->load_wait, 1, 0, true, false);
+                       d->bin_config, d->total_width, d->load_width, d->load_wait, 1, 0, true, false,
+                       d->act_fake_quant, d->weight_fake_quant);
     if (rc) return rc;
     if (pl.wide && !(pl.ZC == 4 || pl.ZC == 8)) {
         set_error("linear: internal planning error (wide accumulation with chunk width %d)", pl.ZC);
@@ -331,10 +346,26 @@ int static_scratch(void **out)
     return REXSC_OK;
 }
 
+// Kept weight streams (REXSC_WSTREAMS_FILL / _VERIFY): one small launch brings the buffer's copy of the weights up to
+// date and stamps the buffer's flag with this call's epoch if anything differed (always, when filling).  The
+// generator launches that follow carry (flag, epoch) and return at once when the stamp is an older one.
+int kept_weights_changed(const ScPlan &pl, const float *w, void *wstreams, int mode, const unsigned long long **guard,
+                         unsigned long long *epoch, hipStream_t stream)
+{
+    REXSC_CHECK_ARG(mode == REXSC_WSTREAMS_FILL || mode == REXSC_WSTREAMS_VERIFY, "weight_streams_valid must be 0, 1 or 2 (got %d)", mode);
+    REXSC_CHECK_ARG(w != nullptr, "null weight pointer");
+    uint8_t *base = (uint8_t *)wstreams;
+    unsigned long long *flag = (unsigned long long *)(base + pl.wstream_off_flag);
+    *epoch = next_epoch();
+    *guard = mode == REXSC_WSTREAMS_VERIFY ? flag : nullptr;
+    return weights_snapshot(w, (float *)(base + pl.wstream_off_snap), pl.w_elems, flag, *epoch,
+                            mode == REXSC_WSTREAMS_FILL, stream);
+}
+
 // The conv op proper: generators, compute, finalize, batch chunk by batch chunk, in `workspace`
 // (device memory of at least pl.total bytes).  wstreams != nullptr: the weight streams and the activation
-// generator's state-plane table live there (pl.wstream_total bytes) instead of in the workspace, and are
-// generated only when wstreams_valid is zero.
+// generator's state-plane table live there (pl.wstream_total bytes) instead of in the workspace;
+// wstreams_valid is one of REXSC_WSTREAMS_*.
 int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const float *w, int16_t *out_pos,
              int16_t *out_neg, int16_t *out_diff, float *out_value, void *wstreams, int wstreams_valid, void *workspace,
              hipStream_t stream)
@@ -352,11 +383,17 @@ int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const f
         if (pl.fold) W2 = (uint32_t *)((uint8_t *)wstreams + pl.wstream_off_w2);
     }
     int rc;
-    if (!wstreams || !wstreams_valid) {
-        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+    if (!wstreams || wstreams_valid != REXSC_WSTREAMS_TRUST) {
+        const unsigned long long *guard = nullptr;
+        unsigned long long epoch = 0;
+        if (wstreams) {
+            rc = kept_weights_changed(pl, w, wstreams, wstreams_valid, &guard, &epoch, stream);
+            if (rc) return rc;
+        }
+        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream, guard, epoch);
         if (rc) return rc;
         if (pl.fold) {
-            rc = fold_weight_streams(Wst, W2, pl.cp.n_slots, pl.fold_KH, pl.fold_KW, pl.wg.O_pad, d->C, stream);
+            rc = fold_weight_streams(Wst, W2, pl.cp.n_slots, pl.fold_KH, pl.fold_KW, pl.wg.O_pad, d->C, stream, guard, epoch);
             if (rc) return rc;
         }
     }
@@ -402,7 +439,7 @@ int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const f
 using namespace rexsc;
 
 extern "C" const char *rexsc_last_error(void) { return g_error; }
-extern "C" int rexsc_version(void) { return 100; }
+extern "C" int rexsc_version(void) { return REXSC_ABI_VERSION; }
 
 extern "C" int rexsc_init(rexsc_stream_t stream)
 {
@@ -467,7 +504,8 @@ extern "C" int rexsc_conv2d_orn_ex(const rexsc_conv_desc *d, const float *x, con
     ScPlan pl;
     int rc = plan_conv(pl, d);
     if (rc) return rc;
-    REXSC_CHECK_ARG(x && (w || (weight_streams && weight_streams_valid)), "null operand pointer");
+    REXSC_CHECK_ARG(x && (w || (weight_streams && weight_streams_valid == REXSC_WSTREAMS_TRUST)), "null operand pointer");
+    REXSC_CHECK_ARG(weight_streams_valid >= 0 && weight_streams_valid <= 2, "weight_streams_valid must be 0, 1 or 2");
     REXSC_CHECK_ARG(out_pos || out_neg || out_diff || out_value, "no output pointer given");
     if (!workspace || workspace_bytes < pl.total) {
         set_error("conv2d: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
@@ -525,8 +563,14 @@ static int run_linear(const ScPlan &pl, const float *x, const float *w, int32_t 
         if (pl.tab_a_words) tab_a = (uint32_t *)((uint8_t *)wstreams + pl.wstream_off_tab);
     }
     int rc;
-    if (!wstreams || !wstreams_valid) {
-        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream);
+    if (!wstreams || wstreams_valid != REXSC_WSTREAMS_TRUST) {
+        const unsigned long long *guard = nullptr;
+        unsigned long long epoch = 0;
+        if (wstreams) {
+            rc = kept_weights_changed(pl, w, wstreams, wstreams_valid, &guard, &epoch, stream);
+            if (rc) return rc;
+        }
+        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream, guard, epoch);
         if (rc) return rc;
     }
     rc = sng_activations(x, A, tab_a, pl.ag, pl.gen_act, stream);
@@ -568,7 +612,8 @@ extern "C" int rexsc_linear_orn_ex(const rexsc_linear_desc *d, const float *x, c
     ScPlan pl;
     int rc = plan_linear(pl, d);
     if (rc) return rc;
-    REXSC_CHECK_ARG(x && out_pos && out_neg && (w || (weight_streams && weight_streams_valid)), "null pointer");
+    REXSC_CHECK_ARG(x && out_pos && out_neg && (w || (weight_streams && weight_streams_valid == REXSC_WSTREAMS_TRUST)), "null pointer");
+    REXSC_CHECK_ARG(weight_streams_valid >= 0 && weight_streams_valid <= 2, "weight_streams_valid must be 0, 1 or 2");
     if (!workspace || workspace_bytes < pl.total) {
         set_error("linear: workspace of %zu bytes needed, %zu given", pl.total, workspace ? workspace_bytes : (size_t)0);
         return REXSC_ERR_WORKSPACE;

@@ -32,8 +32,17 @@ int sng_activations(const float *x, uint32_t *A, const uint32_t *table, const Ac
                     hipStream_t stream);
 // act_table != nullptr: the launch also builds the activation generator's state-plane table
 // (sng_act_table_words() words) for (*act_geo, *act_gp).
+// guard != nullptr: every block first reads *guard and returns at once unless it equals `epoch`
+// (weights_snapshot() writes it): streams and table of an earlier launch stay as they are.
 int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, uint32_t *act_table,
-                const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream);
+                const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream,
+                const unsigned long long *guard = nullptr, unsigned long long epoch = 0);
+
+// Device-side change detection for weight streams kept across calls: compares the n floats of w bit for bit with
+// `snapshot`, copies what differs, and stores `epoch` into *flag when anything did (or when force != 0, which also
+// makes the snapshot a plain copy).  *flag is left alone otherwise.
+int weights_snapshot(const float *w, float *snapshot, size_t n, unsigned long long *flag, unsigned long long epoch,
+                     int force, hipStream_t stream);
 
 // Tap folding for layers whose whole receptive field fits one word (C*KH*KW <= 32, one 32-channel word per pixel):
 //   A2[slot][m]      = OR over taps of A[slot][n][yo*s0+ky][xo*s1+kx] << ((ky*KW+kx)*C),  m = (n, yo, xo)
@@ -41,6 +50,7 @@ int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenP
 // so that popcount(A2 & W2) is the sum over the taps of popcount(A & Wst).
 int fold_activation_streams(const uint32_t *A, uint32_t *A2, int n_slots, long a_stride, long a2_stride, int N, int Hp, int Wp,
                             int Ho, int Wo, int KH, int KW, int s0, int s1, int C, hipStream_t stream);
-int fold_weight_streams(const uint32_t *Wst, uint32_t *W2, int n_slots, int KH, int KW, int O_pad, int C, hipStream_t stream);
+int fold_weight_streams(const uint32_t *Wst, uint32_t *W2, int n_slots, int KH, int KW, int O_pad, int C, hipStream_t stream,
+                        const unsigned long long *guard = nullptr, unsigned long long epoch = 0);
 
 } // namespace rexsc

@@ -636,10 +636,12 @@ constexpr int W_COMBO_CHUNK = 8; // (kx, 64-channel half) combinations whose sta
 template <int ZC, int LB, bool PROG, bool S64>
 __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict__ w, uint32_t *__restrict__ Wst,
                                                          const SeqTable *__restrict__ tables, WeightGeom geo, GenParams gp,
-                                                         int slot_group, int wog, ActTableJob job)
+                                                         int slot_group, int wog, ActTableJob job,
+                                                         const unsigned long long *__restrict__ guard, unsigned long long epoch)
 {
     constexpr int CCH = 32 * ZC;
     constexpr int HALVES = (CCH + 63) / 64;
+    if (guard && *guard != epoch) return; // kept streams are still those of these weights (uniform over the grid)
     extern __shared__ __attribute__((aligned(16))) uint8_t s_dyn[];
     uint8_t *s_seq = s_dyn;
     uint8_t *s_inv = s_dyn + SEQ_LEN;
@@ -842,7 +844,8 @@ int sng_activations(const float *x, uint32_t *A, const uint32_t *table, const Ac
 
 template <int ZC>
 static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, const WeightGeom &geo,
-                         const GenParams &gp, const ActTableJob &job, hipStream_t stream)
+                         const GenParams &gp, const ActTableJob &job, hipStream_t stream, const unsigned long long *guard,
+                         unsigned long long epoch)
 {
     int wog = W_OG_MAX;
     // every block computes the state planes of its (ky, zg) once, so blocks should not be too small;
@@ -879,7 +882,7 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
                                      4.0 * gp.n_slots * geo.KH * geo.ZG * geo.O_pad * 2 * geo.KW * ZC, stream);
     auto launch = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3((unsigned)n_wblocks2), dim3(256), lds, stream, w, Wst, tables, geo, gp, slot_group,
-                           wog, job);
+                           wog, job, guard, epoch);
     };
     auto launch_lb = [&](auto lb_tag) {
         constexpr int LB = decltype(lb_tag)::value;
@@ -903,7 +906,8 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
 }
 
 int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenParams &gp, uint32_t *act_table,
-                const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream)
+                const ActGeom *act_geo, const GenParams *act_gp, hipStream_t stream, const unsigned long long *guard,
+                unsigned long long epoch)
 {
     const SeqTable *tables = nullptr;
     int rc = get_seq_tables(&tables, stream);
@@ -916,12 +920,64 @@ int sng_weights(const float *w, uint32_t *Wst, const WeightGeom &geo, const GenP
         job = act_table_job(act_table, *act_geo, *act_gp);
     }
     switch (geo.ZC) {
-    case 1: return launch_weight<1>(w, Wst, tables, geo, gp, job, stream);
-    case 2: return launch_weight<2>(w, Wst, tables, geo, gp, job, stream);
-    case 4: return launch_weight<4>(w, Wst, tables, geo, gp, job, stream);
-    case 8: return launch_weight<8>(w, Wst, tables, geo, gp, job, stream);
+    case 1: return launch_weight<1>(w, Wst, tables, geo, gp, job, stream, guard, epoch);
+    case 2: return launch_weight<2>(w, Wst, tables, geo, gp, job, stream, guard, epoch);
+    case 4: return launch_weight<4>(w, Wst, tables, geo, gp, job, stream, guard, epoch);
+    case 8: return launch_weight<8>(w, Wst, tables, geo, gp, job, stream, guard, epoch);
     default: set_error("weight SNG: unsupported chunk width %d", geo.ZC); return REXSC_ERR_INVALID;
     }
+}
+
+// ---- change detection for kept weight streams -------------------------------------------------------
+// Bitwise comparison (a NaN equals itself, -0 differs from +0: the streams are a function of the bit pattern's
+// value class only, so this can regenerate needlessly but never miss a change).  Every thread repairs the
+// snapshot elements it finds different; a wave that found any stores the epoch (all writers store the same value).
+__global__ __launch_bounds__(256) void weights_snapshot_kernel(const uint32_t *__restrict__ w, uint32_t *__restrict__ snap,
+                                                               size_t n, unsigned long long *__restrict__ flag,
+                                                               unsigned long long epoch, int force, int vec4)
+{
+    bool diff = false;
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, nthreads = (size_t)gridDim.x * 256;
+    if (vec4) {
+        const size_t n4 = n / 4;
+        const uint4 *w4 = reinterpret_cast<const uint4 *>(w);
+        uint4 *s4 = reinterpret_cast<uint4 *>(snap);
+        for (size_t i = tid; i < n4; i += nthreads) {
+            const uint4 a = w4[i];
+            bool d = true;
+            if (!force) {
+                const uint4 b = s4[i];
+                d = (a.x != b.x) | (a.y != b.y) | (a.z != b.z) | (a.w != b.w);
+            }
+            if (d) { s4[i] = a; diff = true; }
+        }
+        for (size_t i = n4 * 4 + tid; i < n; i += nthreads) {
+            const uint32_t a = w[i];
+            if (force || a != snap[i]) { snap[i] = a; diff = true; }
+        }
+    } else {
+        for (size_t i = tid; i < n; i += nthreads) {
+            const uint32_t a = w[i];
+            if (force || a != snap[i]) { snap[i] = a; diff = true; }
+        }
+    }
+    if (force) diff = true;
+    if (__ballot(diff) != 0ull && (threadIdx.x & 63) == 0) *flag = epoch;
+}
+
+int weights_snapshot(const float *w, float *snapshot, size_t n, unsigned long long *flag, unsigned long long epoch,
+                     int force, hipStream_t stream)
+{
+    REXSC_CHECK_ARG(w && snapshot && flag && n > 0, "weight snapshot: null pointer");
+    const int vec4 = ((uintptr_t)w % 16 == 0) && ((uintptr_t)snapshot % 16 == 0);
+    const size_t per_block = 256 * 4 * 4; // four 16-byte vectors per thread
+    size_t blocks = (n + per_block - 1) / per_block;
+    if (blocks > 2048) blocks = 2048;
+    ProfScope prof("weights_snapshot", 8.0 * n, stream); // w read, snapshot read or written
+    hipLaunchKernelGGL(weights_snapshot_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint32_t *)w,
+                       (uint32_t *)snapshot, n, flag, epoch, force, vec4);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
 }
 
 // ---- tap folding --------------------------------------------------------------------------------
@@ -943,8 +999,10 @@ __global__ __launch_bounds__(256) void fold_act_kernel(const uint32_t *__restric
 }
 
 __global__ __launch_bounds__(256) void fold_weight_kernel(const uint32_t *__restrict__ Wst, uint32_t *__restrict__ W2, int n_slots,
-                                                          int KH, int KW, int O_pad, int C)
+                                                          int KH, int KW, int O_pad, int C,
+                                                          const unsigned long long *__restrict__ guard, unsigned long long epoch)
 {
+    if (guard && *guard != epoch) return;
     // one thread per (slot, o, pol); Wst[slot][ky][o][pol][kx] (one word per pixel and tap)
     const long total = (long)n_slots * O_pad * 2;
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
@@ -971,13 +1029,14 @@ int fold_activation_streams(const uint32_t *A, uint32_t *A2, int n_slots, long a
     return REXSC_OK;
 }
 
-int fold_weight_streams(const uint32_t *Wst, uint32_t *W2, int n_slots, int KH, int KW, int O_pad, int C, hipStream_t stream)
+int fold_weight_streams(const uint32_t *Wst, uint32_t *W2, int n_slots, int KH, int KW, int O_pad, int C, hipStream_t stream,
+                        const unsigned long long *guard, unsigned long long epoch)
 {
     REXSC_CHECK_ARG(C * KH * KW <= 32, "tap folding: receptive field wider than one word");
     const long total = (long)n_slots * O_pad * 2;
     ProfScope prof("fold_weight", 4.0 * total * (KH * KW + 1), stream);
     const int grid = (int)((total + 255) / 256 < 2048 ? (total + 255) / 256 : 2048);
-    hipLaunchKernelGGL(fold_weight_kernel, dim3(grid), dim3(256), 0, stream, Wst, W2, n_slots, KH, KW, O_pad, C);
+    hipLaunchKernelGGL(fold_weight_kernel, dim3(grid), dim3(256), 0, stream, Wst, W2, n_slots, KH, KW, O_pad, C, guard, epoch);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

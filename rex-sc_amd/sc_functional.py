@@ -539,7 +539,7 @@ def conv2d_sc_inference(activation, weight, padding, stride, prec, weight_prec, 
         return _ops.sc_conv2d(activation, weight, bit_length, LFSR_Length, padding, stride,
                               (prec_default, kwargs.get("load_unit", 8), kwargs.get("load_wait_w", 1)), bin_config,
                               gen_config, want_split=False, xnor=_ops.honour_xnor(XNOR), want_value=True,
-                              weight_cache=weight_stream_cache, weight_owner=weight, act_fake_quant=prec,
+                              weight_cache=weight_stream_cache, act_fake_quant=prec,
                               weight_fake_quant=weight_prec)[3]
 
 
@@ -590,9 +590,10 @@ def linear_generic_sc(activation, weight, **kwargs):
 
 
 def linear_sc_inference(activation, weight, prec, weight_stream_cache=None, **kwargs):
-    """Forward value of Linear_Or's default path without autograd: quantise the input, run the SC linear op on the
-    quantised weights and return pos / L - neg / L.  `weight` is the layer's PARAMETER: with a weight_stream_cache
-    its bitstreams (and the quantisation pass that precedes them) are reused until the parameter changes."""
+    """Forward value of Linear_Or's default path without autograd: the SC linear op on the fake-quantised input and
+    weights (the quantisation happens inside the stream generators), returned as pos / L - neg / L.  `weight` is the
+    layer's unquantised PARAMETER: with a weight_stream_cache its bitstreams are kept between calls and regenerated
+    on the device only when its values have changed."""
     bit_length = setvalue_default(kwargs, "bit_length", 128)
     forward = setvalue_default(kwargs, "forward", "or_2")
     generator = setvalue_default(kwargs, "generator", "lfsr")
@@ -603,10 +604,11 @@ def linear_sc_inference(activation, weight, prec, weight_stream_cache=None, **kw
     if bin_config is None or gen_config is None:
         raise ValueError("linear_sc_inference: unsupported forward=%r / generator=%r" % (forward, generator))
     with torch.no_grad():
-        x = quantize(activation, prec=prec)
-        pos, neg = _ops.sc_linear(x, weight, (prec_default, load_unit, load_wait_w), bit_length, LFSR_Length, bin_config,
-                                  gen_config, weight_cache=weight_stream_cache, weight_owner=weight,
-                                  weight_transform=lambda w: quantize(w, prec=prec))
+        if not 0 <= prec <= 16:  # outside what the generators fold: quantise in passes of their own
+            activation, weight, prec = quantize(activation, prec=prec), quantize(weight, prec=prec), None
+        pos, neg = _ops.sc_linear(activation, weight, (prec_default, load_unit, load_wait_w), bit_length, LFSR_Length,
+                                  bin_config, gen_config, weight_cache=weight_stream_cache, act_fake_quant=prec,
+                                  weight_fake_quant=prec)
         # int16 like the CUDA op's outputs (sc_cuda.cpp:101-120), which linear_generic_sc also goes through
         return _ops.sc_counts_to_float(pos.to(torch.int16), neg.to(torch.int16), bit_length)
 

@@ -33,6 +33,15 @@ class Conv2d_Add_Partial(nn.Conv2d):
         self.register_buffer("std_coef", torch.zeros(self.run_args["order"] + 1))
         self._weight_streams = _ops.WeightStreamCache()  # not a buffer: derived data, never part of a state_dict
 
+    def train(self, mode=True):
+        if mode:  # training regenerates the streams on every call: give the kept ones back
+            self._weight_streams.clear()
+        return super(Conv2d_Add_Partial, self).train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._weight_streams.clear()
+        return super(Conv2d_Add_Partial, self)._load_from_state_dict(*args, **kwargs)
+
     def _fn_args(self):
         keys = ("bit_length", "generator", "forward", "load_unit", "load_wait_w", "split_output", "order", "sync")
         return {k: self.run_args[k] for k in keys}
@@ -43,8 +52,9 @@ class Conv2d_Add_Partial(nn.Conv2d):
         else:
             weight_prec = self.run_args["prec"]
         if self.groups == 1 and self.run_args["sync"] == 1 and not torch.is_grad_enabled():
-            # evaluation: SC forward alone, quantisation folded into the generators, weight streams kept while the
-            # parameter does not change (REXSC_WEIGHT_STREAM_CACHE=0 regenerates them on every call)
+            # evaluation: SC forward alone, quantisation folded into the generators, weight streams kept between
+            # calls and regenerated on the device when the weights' values have changed, by whatever route
+            # (REXSC_WEIGHT_STREAM_CACHE=0 regenerates them on every call)
             cache = self._weight_streams if os.environ.get("REXSC_WEIGHT_STREAM_CACHE", "1") != "0" else None
             out = utils_f.conv2d_sc_inference(input, self.weight, self.padding, self.stride, self.run_args["prec"], weight_prec,
                                               weight_stream_cache=cache, **self._fn_args())
@@ -94,6 +104,15 @@ class Linear_Or(nn.Linear):
         self.register_buffer("weight_flag", self.weight.data.clone())
         self._weight_streams = _ops.WeightStreamCache()
 
+    def train(self, mode=True):
+        if mode:
+            self._weight_streams.clear()
+        return super(Linear_Or, self).train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._weight_streams.clear()
+        return super(Linear_Or, self)._load_from_state_dict(*args, **kwargs)
+
     def forward(self, input, prec=7, err=7, generator="lfsr"):
         if self.legacy:
             input.data = utils_f.quantize(input.data, prec=prec)
@@ -101,8 +120,8 @@ class Linear_Or(nn.Linear):
             return utils_f.linear_generic(input, weight, bit_length=2 ** err, forward="full_or", generator=generator)
         keys = ("bit_length", "forward", "generator", "load_unit", "load_wait_w", "sync")
         if self.run_args["sync"] == 1 and not torch.is_grad_enabled() and input.is_cuda:
-            # evaluation: the weight bitstreams (generated from the quantised weights) are kept while the parameter
-            # does not change (REXSC_WEIGHT_STREAM_CACHE=0 regenerates them on every call)
+            # evaluation: the weight bitstreams are kept between calls and regenerated on the device when the
+            # weights' values have changed (REXSC_WEIGHT_STREAM_CACHE=0 regenerates them on every call)
             cache = self._weight_streams if os.environ.get("REXSC_WEIGHT_STREAM_CACHE", "1") != "0" else None
             return utils_f.linear_sc_inference(input, self.weight, self.run_args["prec"], weight_stream_cache=cache,
                                                **{k: self.run_args[k] for k in keys})

@@ -34,7 +34,8 @@ def test_library_exports_every_declared_symbol():
 def test_planning_and_errors_need_no_gpu():
     import _lib
     L = _lib.lib()
-    assert L.rexsc_version() >= 100
+    header = open(os.path.join(ROOT, "include", "rexsc.h")).read()
+    assert L.rexsc_version() == _lib.ABI_VERSION == int(re.search(r"#define REXSC_ABI_VERSION (\d+)", header).group(1))
     d = _lib.ConvDesc(64, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 32, -1, 1, 1, 7, 8, 1, 1, 0)
     assert L.rexsc_conv2d_workspace_bytes(ctypes.byref(d)) > 32 * 64 * 58 * 58 * 2 * 4
     bad = _lib.ConvDesc(64, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 48, -1, 1, 1, 7, 8, 1, 1, 0)  # L=48 unsupported
@@ -47,6 +48,34 @@ def test_planning_and_errors_need_no_gpu():
     assert L.rexsc_linear_workspace_bytes(ctypes.byref(ld)) > 0
     fd = _lib.FixedDesc(2, 8, 6, 6, 4, 3, 3, 1, 1, 1, 1, 0, 5, 24)
     assert L.rexsc_fixed_conv2d_workspace_bytes(ctypes.byref(fd)) > 0
+
+
+def test_descriptor_of_another_abi_is_rejected():
+    """Every descriptor starts with its own size; one built against another header (here: three int32 fields short,
+    the conv descriptor of ABI 100) is refused instead of being read past its end."""
+    import _lib
+    L = _lib.lib()
+    d = _lib.ConvDesc(64, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 32, -1, 1, 1, 7, 8, 1, 1, 0)
+    assert d.struct_size == ctypes.sizeof(_lib.ConvDesc) == 24 * 4
+    d.struct_size -= 12
+    assert L.rexsc_conv2d_workspace_bytes(ctypes.byref(d)) == 0
+    assert b"struct_size" in L.rexsc_last_error()
+    out = (ctypes.c_int64 * 16)()
+    assert L.rexsc_conv2d_plan_info(ctypes.byref(d), out) == -1
+    ld = _lib.LinearDesc(256, 4096, 1024, 64, -1, 1, 1, 7, 8, 1)
+    assert ld.struct_size == 13 * 4 and ld.weight_fake_quant == 0
+    ld.struct_size = 0
+    assert L.rexsc_linear_workspace_bytes(ctypes.byref(ld)) == 0 and b"struct_size" in L.rexsc_last_error()
+    fd = _lib.FixedDesc(2, 8, 6, 6, 4, 3, 3, 1, 1, 1, 1, 0, 5, 24)
+    fd.struct_size += 4
+    assert L.rexsc_fixed_conv2d_workspace_bytes(ctypes.byref(fd)) == 0 and b"struct_size" in L.rexsc_last_error()
+    # the ctypes mirrors have as many int32 fields as the header's structures
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "rexsc.h")).read(), flags=re.S)
+    for name, cls in (("rexsc_conv_desc", _lib.ConvDesc), ("rexsc_linear_desc", _lib.LinearDesc),
+                      ("rexsc_fixed_desc", _lib.FixedDesc)):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, flags=re.S).group(1)
+        fields = [f.strip() for decl in re.findall(r"int32_t([^;]*);", body) for f in decl.split(",")]
+        assert fields == [f[0] for f in cls._fields_], name
 
 
 def test_philox_known_answers():

@@ -71,26 +71,128 @@ def test_weight_stream_cache_reuse_and_invalidation():
     assert (cache.hits, cache.misses) == (1, 1)
     for r in (a, b):
         assert torch.equal(r[0], want[0]) and torch.equal(r[1], want[1])
-    # other activations, same weights: the cached streams serve
+    # other activations, same weights: the kept streams serve
     x2 = torch.roll(xt, 1, 0).contiguous(memory_format=torch.channels_last)
     c = _ops.sc_conv2d(x2, *args[1:], weight_cache=cache)
     assert cache.hits == 2 and torch.equal(c[0], _ops.sc_conv2d(x2, *args[1:])[0])
-    # an in-place update of the weights bumps the version counter: regenerated
+    # an in-place update of the weights: same buffer, regenerated on the device
     with torch.no_grad():
         wt.mul_(-0.5)
     d = _ops.sc_conv2d(*args, weight_cache=cache)
-    assert cache.misses == 2
+    assert cache.misses == 1
     want2 = _ops.sc_conv2d(*args)
     assert torch.equal(d[0], want2[0]) and torch.equal(d[1], want2[1]) and not torch.equal(d[0], want[0])
+    # in-place edits through .data, which neither move the storage nor bump the version counter
+    version = wt._version
+    wt.data.clamp_(-0.25, 0.125)
+    assert wt._version == version
+    d2 = _ops.sc_conv2d(*args, weight_cache=cache)
+    want3 = _ops.sc_conv2d(*args)
+    assert torch.equal(d2[0], want3[0]) and torch.equal(d2[1], want3[1]) and not torch.equal(d2[0], want2[0])
     # new storage behind the same tensor object
     wt.data = torch.from_numpy(w).cuda()
     e = _ops.sc_conv2d(*args, weight_cache=cache)
-    assert cache.misses == 3 and torch.equal(e[0], want[0])
+    assert cache.misses == 1 and torch.equal(e[0], want[0])
     # another batch size is another descriptor (its own entry); both stay valid
     f = _ops.sc_conv2d(xt[:1].contiguous(memory_format=torch.channels_last), *args[1:], weight_cache=cache)
-    assert cache.misses == 4 and torch.equal(f[0], want[0][:1])
+    assert cache.misses == 2 and torch.equal(f[0], want[0][:1])
     g = _ops.sc_conv2d(*args, weight_cache=cache)
-    assert cache.hits == 3 and torch.equal(g[0], want[0])
+    assert cache.misses == 2 and torch.equal(g[0], want[0])
+
+
+def test_kept_weight_streams_are_used_until_the_weights_change():
+    """The device-side check really skips generation while the weights are unchanged (the streams in the buffer are
+    what the call computes with -- shown by wiping them) and regenerates after a single-element edit."""
+    import _ops
+    cfg = (2, 64, 10, 10, 32, 3, 1, 32, 1, False)
+    x, w, xt, wt = _operands(cfg, seed=9)
+    cache = _ops.WeightStreamCache()
+    args = (xt, wt, 32, -1, (1, 1), (1, 1), (7, 8, 1), 1, 1)
+    want = _ops.sc_conv2d(*args)
+    assert torch.equal(_ops.sc_conv2d(*args, weight_cache=cache)[0], want[0]) and int(want[0].max()) > 0
+    (buf,) = cache.entries.values()
+    keep = (wt.numel() * 4 + 255) // 256 * 256 + 256   # the copy of the weights and the change flag close the buffer
+    buf[:buf.numel() - keep].zero_()                    # wipe streams and tables
+    wiped = _ops.sc_conv2d(*args, weight_cache=cache)
+    assert int(wiped[0].abs().max()) == 0 and int(wiped[1].abs().max()) == 0   # nothing was regenerated
+    wt.data.view(-1)[-1] += 0.25                        # one element, through .data
+    again = _ops.sc_conv2d(*args, weight_cache=cache)
+    want2 = _ops.sc_conv2d(*args)
+    assert torch.equal(again[0], want2[0]) and torch.equal(again[1], want2[1])
+    assert torch.equal(_ops.sc_conv2d(*args, weight_cache=cache)[0], want2[0])
+
+
+def _oracle_layer_value(x, w, prec, L, padding, stride, cla):
+    xq, wq = orc.quantize(x.cpu().numpy(), prec), orc.quantize(w.cpu().numpy(), prec)
+    opos, oneg = orc.conv2d_generic_general_split(xq, wq, L, -1, 16, padding, stride, (7, 8, 1), 1, 1,
+                                                  channels_last_activation=cla)
+    return opos.astype(np.float32) / np.float32(L) - oneg.astype(np.float32) / np.float32(L)
+
+
+def _edit_weight_data(weight, edit):
+    if edit == "clamp":          # literally the reference's line (the layers' quantisation clamps tighter anyway)
+        weight.data.clamp_(-1, 0.999)
+    elif edit == "clamp_tight":  # a clamp that does change the quantised weights
+        weight.data.clamp_(-0.25, 0.125)
+    else:
+        weight.data.mul_((torch.rand_like(weight) < 0.5).float())
+
+
+@pytest.mark.parametrize("edit", ["clamp", "clamp_tight", "mask"])
+def test_evaluation_after_inplace_data_edit_conv(edit):
+    """eval -> weight.data.<op>_() -> eval (the reference's own loop clamps this way, utils_own.py:187-190):
+    the second evaluation must be that of the NEW weights, against the oracle."""
+    from sc_layers import Conv2d_Add_Partial
+    torch.manual_seed(11)
+    layer = Conv2d_Add_Partial(40, 24, kernel_size=3, padding=1, bias=False, forward="or_2", err=5).cuda().eval()
+    with torch.no_grad():
+        layer.weight.mul_(6.0)   # some weights beyond +-1, so that the clamp changes values
+    x = (torch.rand(2, 40, 9, 9, device="cuda") * 1.1 - 0.05).contiguous(memory_format=torch.channels_last)
+    with torch.no_grad():
+        y1 = layer(x)
+    assert np.array_equal(y1.cpu().numpy(), _oracle_layer_value(x, layer.weight.data, 7, 32, (1, 1), (1, 1), True))
+    version = layer.weight._version
+    _edit_weight_data(layer.weight, edit)
+    assert layer.weight._version == version
+    with torch.no_grad():
+        y2 = layer(x)
+    assert (layer._weight_streams.hits, layer._weight_streams.misses) == (1, 1)
+    assert np.array_equal(y2.cpu().numpy(), _oracle_layer_value(x, layer.weight.data, 7, 32, (1, 1), (1, 1), True))
+    assert edit == "clamp" or not torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("edit", ["clamp", "clamp_tight", "mask"])
+def test_evaluation_after_inplace_data_edit_linear(edit):
+    import sc_functional as uf
+    from sc_layers import Linear_Or
+    torch.manual_seed(12)
+    layer = Linear_Or(96, 40, bias=False, forward="or_2", err=6).cuda().eval()
+    with torch.no_grad():
+        layer.weight.mul_(12.0)
+    x = torch.rand(5, 96, device="cuda") * 1.1 - 0.05
+
+    def oracle_value():
+        xq = orc.quantize(x.cpu().numpy(), 7)
+        wq = orc.quantize(layer.weight.data.cpu().numpy(), 7)
+        pos, neg = orc.linear_generic_general(xq, wq, (7, 8, 1), 64, -1, 1, 1, True, False)
+        return (pos.astype(np.float32) - neg.astype(np.float32)) / 64
+
+    with torch.no_grad():
+        y1 = layer(x)
+    assert np.array_equal(y1.cpu().numpy(), oracle_value())
+    _edit_weight_data(layer.weight, edit)
+    with torch.no_grad():
+        y2 = layer(x)
+    assert (layer._weight_streams.hits, layer._weight_streams.misses) == (1, 1)
+    assert np.array_equal(y2.cpu().numpy(), oracle_value()) and (edit == "clamp" or not torch.equal(y1, y2))
+    # entering training mode and loading a state dict give the kept streams back
+    layer.train()
+    assert not layer._weight_streams.entries
+    layer.eval()
+    with torch.no_grad():
+        layer(x)
+    layer.load_state_dict(layer.state_dict())
+    assert not layer._weight_streams.entries
 
 
 @pytest.mark.parametrize("sng_mode", ["1", "2"])
@@ -135,19 +237,20 @@ def test_layer_evaluation_path_equals_training_forward(monkeypatch):
     opt.step()
     with torch.no_grad():
         y3 = layer(x)
-    assert layer._weight_streams.misses == 2
+    assert layer._weight_streams.misses == 1  # same buffer: the device noticed the new values
     assert torch.equal(y3, layer(x.clone().requires_grad_(True)).detach()) and not torch.equal(y3, y1)
     # switched off: same values, nothing cached
     monkeypatch.setenv("REXSC_WEIGHT_STREAM_CACHE", "0")
+    calls = layer._weight_streams.hits + layer._weight_streams.misses
     with torch.no_grad():
         y4 = layer(x)
-    assert torch.equal(y4, y3) and layer._weight_streams.misses == 2
+    assert torch.equal(y4, y3) and layer._weight_streams.hits + layer._weight_streams.misses == calls
     assert "_weight_streams" not in layer.state_dict()
 
 
 def test_linear_layer_evaluation_path_and_weight_stream_cache(monkeypatch):
-    """Linear_Or under no_grad: same values as its training forward, weight bitstreams generated once per weight
-    version, for any batch size, and straight against the oracle on the quantised operands."""
+    """Linear_Or under no_grad: same values as its training forward, weight bitstreams kept in one buffer for any
+    batch size, and straight against the oracle on the quantised operands."""
     import sc_functional as uf
     from sc_layers import Linear_Or
     torch.manual_seed(6)
@@ -171,12 +274,13 @@ def test_linear_layer_evaluation_path_and_weight_stream_cache(monkeypatch):
     opt.step()
     with torch.no_grad():
         y3 = layer(x)
-    assert layer._weight_streams.misses == 2
+    assert layer._weight_streams.misses == 1
     assert torch.equal(y3, layer(x.clone().requires_grad_(True)).detach()) and not torch.equal(y3, y1)
     monkeypatch.setenv("REXSC_WEIGHT_STREAM_CACHE", "0")
+    calls = layer._weight_streams.hits + layer._weight_streams.misses
     with torch.no_grad():
         y4 = layer(x)
-    assert torch.equal(y4, y3) and layer._weight_streams.misses == 2
+    assert torch.equal(y4, y3) and layer._weight_streams.hits + layer._weight_streams.misses == calls
     assert "_weight_streams" not in layer.state_dict()
 
 
