@@ -931,6 +931,285 @@ __global__ __launch_bounds__(256, 2) void fixed_fused_kernel(const float *__rest
     if (pending >= 0) store_item(pending);
 }
 
+// ---- single pass for small planes: the reduction split over the waves of a block ---------------------------------
+// 3x3 / stride 1 / padding 1 layers whose planes are small (14x14, 7x7) have many channels and few pixels: a block that
+// walks the whole reduction is long, and there are too few of them to hide their load latency.  Here a block still owns a
+// tile of output pixels (TH rows x W columns of one image, at most 64 pixels) and 64 output channels, but its four waves
+// take a quarter of the 32-channel groups each and work on it independently of one another -- nothing is shared, so there
+// is no barrier inside the reduction: a wave reads the float32 activations of its groups from the NCHW tensor, rounds /
+// clamps / packs them to int8 into its own LDS region (halo included; LDS operations of one wave execute in order, so the
+// wave may read what it has just written), and takes its weights -- int8 values tiled by fixed_pack_w_values in the MFMA
+// operand order -- straight from L2 into registers, a kernel row at a time, two rows ahead of their use; the parity operand
+// of the weights is derived in registers.  The four partial tiles meet in LDS at the end (two exchange rounds, after which
+// every wave holds one quarter of the tile and stores it).  Blocks are four times shorter and four times more numerous than
+// with the whole reduction per block, the int8 copy of the activations never reaches HBM and nothing is added atomically.
+struct KsplitParams {
+    int N, C, H, W, O, O_pad;
+    int pairs;            // 32-channel groups, ceil(C / 32)
+    int TH, tiles_y;      // tile: TH output rows x W columns; tiles per image
+    int o_tiles, n_items; // one block per (image, tile, output-channel tile)
+    float P2;
+};
+
+// weights -> wv[otile][pair][h][tap][o 0..63]: 16-byte entries (16 channels of one tap and output channel), values only.
+// One thread per entry, tap fastest: the threads of one (o, 16-channel block) read one contiguous run of the OIHW tensor.
+__global__ __launch_bounds__(256) void fixed_pack_w_values(const float *__restrict__ w, int8_t *__restrict__ wv, int O, int C,
+                                                           int O_pad, int pairs, float P2)
+{
+    const unsigned total = (unsigned)O_pad * pairs * 2 * 9;
+    const unsigned i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const unsigned tap = i % 9, co = i / 9;
+    const unsigned cb = co % (unsigned)(pairs * 2), o = co / (unsigned)(pairs * 2);
+    float f[16];
+    const float *src = w + ((long)o * C + cb * 16) * 9 + tap;
+    if ((int)o < O && (int)(cb * 16 + 16) <= C) {
+#pragma unroll
+        for (int k = 0; k < 16; k++) f[k] = src[k * 9];
+    } else {
+#pragma unroll
+        for (int k = 0; k < 16; k++) f[k] = ((int)o < O && (int)(cb * 16) + k < C) ? src[k * 9] : 0.f;
+    }
+    uint32_t vals[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const int q = quant_round_pos(f[k], P2) - quant_round_neg(f[k], P2); // signed
+        vals[k >> 2] |= (uint32_t)(uint8_t)(int8_t)q << (8 * (k & 3));
+    }
+    const unsigned otile = o / 64, ol = o % 64, pair = cb / 2, h = cb % 2;
+    reinterpret_cast<uint4 *>(wv)[((((long)otile * pairs + pair) * 2 + h) * 9 + tap) * 64 + ol] = make_uint4(vals[0], vals[1], vals[2], vals[3]);
+}
+
+// A wave-uniform 64-bit offset the compiler has to materialise in scalar registers where it stands: it can then not be
+// folded into loop-invariant per-lane address arithmetic (which would keep a 64-bit address pair alive per load).
+__device__ __forceinline__ long opaque_uniform(long v)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)((unsigned long)v >> 32));
+    asm volatile("" : "+s"(lo), "+s"(hi));
+    return (long)(((unsigned long)hi << 32) | lo);
+#else
+    return v;
+#endif
+}
+
+// AR: rounds of 64 (half, tile row incl. halo rows, column) entries that cover the wave's activation tile.
+template <int AR>
+__global__ __launch_bounds__(256, 2) void fixed_ksplit_kernel(const float *__restrict__ x, const v4i *__restrict__ wv,
+                                                             int32_t *__restrict__ out, KsplitParams p)
+{
+    constexpr int PB = 2; // 32-pixel blocks per tile
+    extern __shared__ __attribute__((aligned(16))) uint8_t s_raw[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int j = lane & 31, h = lane >> 5;
+    const int Wp = p.W + 2, RP = p.TH + 2, NPP = RP * Wp; // padded tile
+    v4i *s_a = reinterpret_cast<v4i *>(s_raw) + wave * (2 * NPP); // this wave's region: [half][padded pixel]
+    // blocks of one XCD (ids b, b + 8, ...) take consecutive items: the output-channel tiles of one pixel tile
+    const int G = gridDim.x;
+    const int bid = (G % 8 == 0) ? (int)(blockIdx.x % 8) * (G / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x;
+    const int otile = bid % p.o_tiles;
+    const int tl = bid / p.o_tiles;
+    const int ty = tl % p.tiles_y, n = tl / p.tiles_y;
+    const int y0 = ty * p.TH;
+    const long plane = (long)p.H * p.W;
+
+    // the whole region starts as zeros: halo columns, rows outside the image and channels beyond C stay that way
+    for (int e = lane; e < 2 * NPP; e += 64) s_a[e] = (v4i){0, 0, 0, 0};
+
+    // this lane's entries of the tile: (half, padded row, column) -> element offset from x (32 bits: the host checks the
+    // tensor's size), LDS index and half packed into one word (bit 31: half; negative offset: nothing to load)
+    const int RW = RP * p.W;
+    int e_off[AR], e_lds[AR];
+#pragma unroll
+    for (int a = 0; a < AR; a++) {
+        const int e = a * 64 + lane;
+        const int hh = e >= RW ? 1 : 0;
+        const int rem = e - hh * RW;
+        const int r = rem / p.W, c = rem - r * p.W;
+        const int y = y0 - 1 + r;
+        const bool ok = e < 2 * RW && y >= 0 && y < p.H;
+        e_lds[a] = (hh * NPP + r * Wp + c + 1) | (hh << 30);
+        e_off[a] = ok ? (int)(((long)n * p.C + hh * 16) * plane + (long)y * p.W + c) : -1;
+    }
+    // this lane's output pixels
+    int abase[PB];
+#pragma unroll
+    for (int pb = 0; pb < PB; pb++) {
+        const int t = pb * 32 + j;
+        const int r = t / p.W, c = t - r * p.W;
+        abase[pb] = (r < p.TH) ? r * Wp + c : 0;
+    }
+
+    const int per = (p.pairs + 3) / 4;
+    const int g_begin = min(p.pairs, wave * per), g_end = min(p.pairs, g_begin + per);
+    const int n_rows = (g_end - g_begin) * 3;
+
+    v16i acc[2][PB];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < PB; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0;
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    const float top = p.P2 - 1.f;
+
+    // Rounds 0 .. PF-1 of a group's entries are requested one group ahead and wait in registers; a fourth round (tiles
+    // with more than 192 entries) is loaded when the group is converted, reusing the same registers.
+    constexpr int PF = AR < 3 ? AR : 3;
+    float f[PF][16];
+    auto load_round = [&](int g, int a, float (&dst)[16]) __attribute__((always_inline)) {
+        // wave-uniform byte offset of (group, channel k) + this lane's 32-bit byte offset
+        const char *xc = reinterpret_cast<const char *>(x);
+        if (p.C - g * 32 >= 32) { // a whole group (wave-uniform): every lane loads, lanes without an entry re-read offset 0
+            const uint32_t off = e_off[a] >= 0 ? (uint32_t)e_off[a] * 4u : 0u;
+#pragma unroll
+            for (int k = 0; k < 16; k++)
+                dst[k] = *reinterpret_cast<const float *>(xc + opaque_uniform(((long)g * 32 + k) * plane * 4) + off);
+        } else { // the channel tail of the last group
+            const int kmax = e_off[a] >= 0 ? p.C - g * 32 - (e_lds[a] >> 30) * 16 : 0;
+            const uint32_t off = (uint32_t)e_off[a] * 4u;
+#pragma unroll
+            for (int k = 0; k < 16; k++)
+                dst[k] = k < kmax ? *reinterpret_cast<const float *>(xc + opaque_uniform(((long)g * 32 + k) * plane * 4) + off) : 0.f;
+        }
+    };
+    auto convert_round = [&](int a, const float (&src)[16]) __attribute__((always_inline)) { // int8, round half to even, clamp to [0, P2 - 1] -> LDS
+        uint32_t wds[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int k = 0; k < 16; k++)
+            wds[k >> 2] = __builtin_amdgcn_cvt_pk_u8_f32(fminf(src[k] * p.P2, top), k & 3, wds[k >> 2]);
+        if (e_off[a] >= 0) s_a[e_lds[a] & 0xffff] = (v4i){(int)wds[0], (int)wds[1], (int)wds[2], (int)wds[3]};
+    };
+    auto issue_acts = [&](int g) __attribute__((always_inline)) {
+#pragma unroll
+        for (int a = 0; a < PF; a++) load_round(g, a, f[a]);
+    };
+    // weight rows (group, ky) run through a ring of three register sets, two rows ahead of their use
+    v4i wr[3][2][3]; // [slot][output-channel half][kx]
+    const v4i *wbase = wv + ((long)otile * p.pairs * 2 + h) * (9 * 64) + j;
+    auto load_row = [&](int r, v4i (&dst)[2][3]) __attribute__((always_inline)) {
+        r = r < n_rows ? r : n_rows - 1; // past the end: re-read the last row (harmless)
+        const int g = g_begin + r / 3, ky = r - (r / 3) * 3;
+        const v4i *src = wbase + (long)g * (2 * 9 * 64) + ky * 3 * 64;
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) { dst[0][kx] = src[kx * 64]; dst[1][kx] = src[kx * 64 + 32]; }
+    };
+    if (n_rows > 0) {
+        issue_acts(g_begin);
+        load_row(0, wr[0]);
+        load_row(1, wr[1]);
+    }
+    for (int g = g_begin; g < g_end; g++) {
+        // activations of this group: registers -> int8 -> LDS
+#pragma unroll
+        for (int a0 = 0; a0 < AR; a0 += PF) {
+            if (a0 > 0) {
+                __builtin_amdgcn_sched_barrier(0); // not before the previous rounds have left these registers
+#pragma unroll
+                for (int a = 0; a < PF; a++) if (a0 + a < AR) load_round(g, a0 + a, f[a]);
+            }
+#pragma unroll
+            for (int a = 0; a < PF; a++) if (a0 + a < AR) convert_round(a0 + a, f[a]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (g + 1 < g_end) issue_acts(g + 1);
+        // other lanes of this wave read what this lane wrote: LDS executes a wave's operations in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int r_base = (g - g_begin) * 3;
+        const v4i *sa = s_a + h * NPP;
+#pragma unroll
+        for (int ky = 0; ky < 3; ky++) {
+            load_row(r_base + ky + 2, wr[(ky + 2) % 3]);
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++) {
+                const v4i a0 = wr[ky][0][kx], a1 = wr[ky][1][kx];
+                const v4i q0 = weight_parities(a0), q1 = weight_parities(a1);
+#pragma unroll
+                for (int pb = 0; pb < PB; pb++) {
+                    const v4i b = sa[abase[pb] + ky * Wp + kx];
+                    const v4i par = b & ones;
+                    acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, b, acc[0][pb], 0, 0, 0);
+                    acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, b, acc[1][pb], 0, 0, 0);
+                    acc[0][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q0, par, acc[0][pb], 0, 0, 0);
+                    acc[1][pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(q1, par, acc[1][pb], 0, 0, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // The four partial tiles meet in LDS.  Round A: waves 0/1 and 2/3 exchange output-channel halves (even waves keep
+    // half 0); round B: waves 0/2 and 1/3 exchange pixel blocks (waves 0, 1 keep block 0).  Afterwards wave w holds the
+    // finished quarter (half w & 1, pixel block w >> 1).
+    __syncthreads(); // every wave is done with its activation region, which the exchange buffers overlay
+    int *s_red = reinterpret_cast<int *>(s_raw);
+    v16i keep[PB];
+    {
+        int *mine = s_red + wave * (PB * 16 * 64) + lane;
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mine[(pb * 16 + r) * 64] = (wave & 1) ? acc[0][pb][r] : acc[1][pb][r];
+        __syncthreads();
+        const int *theirs = s_red + (wave ^ 1) * (PB * 16 * 64) + lane;
+#pragma unroll
+        for (int pb = 0; pb < PB; pb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) keep[pb][r] = ((wave & 1) ? acc[1][pb][r] : acc[0][pb][r]) + theirs[(pb * 16 + r) * 64];
+        __syncthreads();
+    }
+    v16i fin;
+    {
+        int *mine = s_red + wave * (16 * 64) + lane;
+#pragma unroll
+        for (int r = 0; r < 16; r++) mine[r * 64] = (wave & 2) ? keep[0][r] : keep[1][r];
+        __syncthreads();
+        const int *theirs = s_red + (wave ^ 2) * (16 * 64) + lane;
+#pragma unroll
+        for (int r = 0; r < 16; r++) fin[r] = ((wave & 2) ? keep[1][r] : keep[0][r]) + theirs[r * 64];
+    }
+    const int a_fin = wave & 1, pb_fin = wave >> 1;
+    const int t = pb_fin * 32 + j;
+    const int row = t / p.W, col = t - row * p.W;
+    const int y = y0 + row;
+    if (row < p.TH && y < p.H) {
+        const int o_first = otile * 64 + a_fin * 32 + 4 * h;
+        int32_t *o0 = out + ((long)n * p.O + o_first) * plane + (long)y * p.W + col;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int ol = 8 * (r / 4) + (r % 4);
+            if (o_first + ol < p.O) o0[(long)ol * plane] = fin[r];
+        }
+    }
+}
+
+// Tile choice of the split-reduction kernel; false when the shape is not one it handles.
+static bool ksplit_plan(const FixedParams &p, int O_pad, KsplitParams &k, int &AR)
+{
+    if (p.KH != 3 || p.KW != 3 || p.s0 != 1 || p.s1 != 1 || p.pad_h != 1 || p.pad_w != 1) return false;
+    if (p.W > 64 || O_pad % 64 != 0) return false;
+    k.N = p.N; k.C = p.C; k.H = p.H; k.W = p.W; k.O = p.O; k.O_pad = O_pad; k.P2 = p.P2;
+    k.pairs = ceil_div(p.C, 32);
+    k.o_tiles = O_pad / 64;
+    int th = 64 / p.W;
+    if (th > p.H) th = p.H;
+    while (th > 1 && 2 * (th + 2) * p.W > 4 * 64) th--; // at most four rounds of tile entries per lane
+    if (th < 1 || 2 * (th + 2) * p.W > 4 * 64) return false;
+    k.TH = th;
+    k.tiles_y = ceil_div(p.H, th);
+    const long items = (long)p.N * k.tiles_y * k.o_tiles;
+    if (items >= (1L << 31)) return false;
+    if ((long)p.N * p.C * p.H * p.W >= (1L << 30)) return false; // 32-bit byte offsets inside the activation tensor
+    k.n_items = (int)items;
+    AR = ceil_div(2 * (th + 2) * p.W, 64);
+    return true;
+}
+
 static int tune_flag(const char *name, int dflt)
 {
     const char *e = getenv(name);
@@ -1081,7 +1360,35 @@ extern "C" int rexsc_fixed_conv2d(const rexsc_fixed_desc *d, const float *x, con
         // the two-pass path spends its time on); on small planes with many channels its blocks are too few and too
         // long to hide their load latency, and the two-pass path stays ahead.  REXSC_TUNE_FIXED_FUSED: 0 never, 2 wherever it can.
         const int fused_mode = tune_flag("REXSC_TUNE_FIXED_FUSED", 1);
-        if (fused_mode && fused_plan(p, q.O_pad, fp) && (fused_mode == 2 || p.H * p.W >= 512)) {
+        // Planes that one 64-pixel tile covers (7x7) with at least eight 32-channel groups: the single pass whose waves split
+        // the reduction (measured 39 us against 43 for the two passes on 512 x 7 x 7, batch 64; on 14 x 14 planes, four tiles
+        // per image, it loses by 3 us).  REXSC_TUNE_FIXED_FUSED: 3 wherever it can run, 0 / 2 never.
+        KsplitParams kp;
+        int ks_ar = 0;
+        if ((fused_mode == 1 || fused_mode == 3) && ksplit_plan(p, q.O_pad, kp, ks_ar) &&
+            (fused_mode == 3 || (p.H * p.W <= 64 && kp.pairs >= 8))) {
+            {
+                ProfScope prof("fixed_pack_weights", 4.0 * p.O * p.C * 9 + 16.0 * q.O_pad * kp.pairs * 2 * 9, stream);
+                const long threads = (long)q.O_pad * kp.pairs * 2 * 9;
+                hipLaunchKernelGGL(fixed_pack_w_values, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, w, wq16,
+                                   p.O, p.C, q.O_pad, kp.pairs, p.P2);
+                REXSC_CHECK_HIP(hipGetLastError());
+            }
+            ProfScope prof("fixed_conv_ksplit", io_bytes, stream);
+            const int NPP = (kp.TH + 2) * (kp.W + 2);
+            size_t lds = (size_t)4 * 2 * NPP * 16;          // the waves' activation regions ...
+            if (lds < 4 * 2 * 16 * 64 * 4) lds = 4 * 2 * 16 * 64 * 4; // ... overlaid by the exchange buffers (32 KB)
+            const v4i *wvp = reinterpret_cast<const v4i *>(wq16);
+            switch (ks_ar) {
+            case 1: hipLaunchKernelGGL((fixed_ksplit_kernel<1>), dim3(kp.n_items), dim3(256), lds, stream, x, wvp, out, kp); break;
+            case 2: hipLaunchKernelGGL((fixed_ksplit_kernel<2>), dim3(kp.n_items), dim3(256), lds, stream, x, wvp, out, kp); break;
+            case 3: hipLaunchKernelGGL((fixed_ksplit_kernel<3>), dim3(kp.n_items), dim3(256), lds, stream, x, wvp, out, kp); break;
+            default: hipLaunchKernelGGL((fixed_ksplit_kernel<4>), dim3(kp.n_items), dim3(256), lds, stream, x, wvp, out, kp); break;
+            }
+            REXSC_CHECK_HIP(hipGetLastError());
+            return REXSC_OK;
+        }
+        if (fused_mode && fused_mode != 3 && fused_plan(p, q.O_pad, fp) && (fused_mode == 2 || p.H * p.W >= 512)) {
             const int NPP = fp.NI * (fp.TH + 2) * (fp.W + 2);
             const int PBT = ceil_div(fp.NI * fp.TH * fp.W, 32);
             const int AR = ceil_div(2 * NPP, 256);

@@ -250,20 +250,23 @@ FUSED_FIXED = [
     (3, 40, 12, 36, 70),    # rows of a multiple of four pixels (16-byte loads), ragged row tiles, two output tiles
     (2, 33, 10, 16, 64),    # 16-byte loads with a channel tail of one
     (600, 8, 4, 8, 8),      # small planes of a multiple of four pixels per row: two images per tile with 16-byte loads
+    (3, 130, 14, 14, 70),   # five channel groups over four waves (2, 2, 1, 0), channel tail of two, ragged row tiles
+    (2, 256, 14, 14, 256),  # config-4 stage 3 at batch 2
 ]
 
 
-@pytest.mark.parametrize("path", ["planner", "single_pass", "single_pass_tiled_weights", "two_pass"])
+@pytest.mark.parametrize("path", ["planner", "single_pass", "single_pass_tiled_weights", "two_pass", "split_reduction"])
 @pytest.mark.parametrize("cfg", FUSED_FIXED, ids=lambda c: "_".join(str(v) for v in c))
 def test_fixed_fused_shapes_and_out_of_range_operands(cfg, path, monkeypatch):
     """Activations below zero, above one, at rounding ties and near-ties; weights likewise.  Once with the
     library's own choice between the single-pass and the two-pass MFMA path, once with each forced (the single
-    pass also without its weights-in-LDS variant)."""
+    pass also without its weights-in-LDS variant, and the single pass whose waves split the reduction wherever its
+    tiling exists -- rows of at most 64 pixels; other shapes fall through to the two passes)."""
     import fixed_extension_cuda
     N, C, H, W, O = cfg
     print("fixed fused", cfg, path, flush=True)
     if path != "planner":
-        monkeypatch.setenv("REXSC_TUNE_FIXED_FUSED", "0" if path == "two_pass" else "2")
+        monkeypatch.setenv("REXSC_TUNE_FIXED_FUSED", {"two_pass": "0", "split_reduction": "3"}.get(path, "2"))
     if path == "single_pass_tiled_weights":   # never the variant that keeps all weights in LDS
         monkeypatch.setenv("REXSC_TUNE_FIXED_WS", "0")
     rng = np.random.default_rng(sum(cfg))
