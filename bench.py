@@ -143,6 +143,10 @@ def main():
     total_mac = sum(layer_macs(N, C, H, O, K, s) for (C, H, O, K, s) in shapes)
 
     def step():
+        """The 19 layers through the reference's own entry point, one call after the other.  (Generating every layer's
+        weight bitstreams on a second stream while earlier layers compute -- rexsc_conv2d_prepare_weights -- was
+        measured here and lost: 10.43 ms against 10.35, the generators' blocks displace blocks of the VALU-bound
+        compute kernel.)"""
         for (x, w, K, s) in layers:
             sc_extension_cuda.conv2d_generic_general_split_acc(
                 x, w, L, -1, 16, (K // 2, K // 2), (s, s), (7, 8, 1), OR_N - 1, 1, True, False)

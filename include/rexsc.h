@@ -116,6 +116,15 @@ int rexsc_conv2d_orn_ex(const rexsc_conv_desc *d, const float *x, const float *w
                         void *weight_streams, size_t weight_streams_bytes, int weight_streams_valid,
                         void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
 
+/* The weight half of rexsc_conv2d_orn_ex on its own (no counterpart in the reference, whose conv2d_generic_general
+ * expands the weights inside every call, sc_conv.cpp:432-450): fills weight_streams as a call in mode
+ * REXSC_WSTREAMS_FILL does and returns; the conv call proper follows in mode REXSC_WSTREAMS_TRUST on a stream ordered
+ * after this one (or, when keep_weight_copy != 0 also stored the copy of w that mode compares with, in mode _VERIFY).
+ * A layer's weight streams depend on its weights alone, so a caller can have them generated on a second stream while
+ * the previous layer still computes. */
+int rexsc_conv2d_prepare_weights(const rexsc_conv_desc *d, const float *w, void *weight_streams,
+                                 size_t weight_streams_bytes, int keep_weight_copy, rexsc_stream_t stream);
+
 /* The same op for callers that cannot allocate device memory or hand over a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
  * reference.  The workspace is a static device array inside the library

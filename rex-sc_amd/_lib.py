@@ -65,6 +65,7 @@ SIGNATURES = {
     "rexsc_conv2d_orn": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "rexsc_conv2d_weight_streams_bytes": (_sz, [ctypes.POINTER(ConvDesc)]),
     "rexsc_conv2d_orn_ex": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _int, _vp, _sz, _vp]),
+    "rexsc_conv2d_prepare_weights": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _sz, _int, _vp]),
     "rexsc_conv2d_orn_noalloc": (_int, [ctypes.POINTER(ConvDesc), _vp, _vp, _vp, _vp, _vp, _vp]),
     "rexsc_linear_workspace_bytes": (_sz, [ctypes.POINTER(LinearDesc)]),
     "rexsc_linear_orn": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),

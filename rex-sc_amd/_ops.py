@@ -119,30 +119,81 @@ class WeightStreamCache:
         self.entries.clear()
 
 
-def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
-              want_split=True, want_diff=False, xnor=False, want_value=False, weight_cache=None,
-              act_fake_quant=None, weight_fake_quant=None):
-    """SC conv2d on the HIP path.  padding=(p0,p1): p0 pads the LAST axis, p1 axis 2, as the
-    reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2.
-    -> (pos, neg, diff) int16, plus the float32 tensor pos / L - neg / L as a fourth element when want_value.
-    weight_cache: a WeightStreamCache that keeps w's bitstreams between calls (the device checks on every call that
-    they still belong to w's values).  act_fake_quant / weight_fake_quant: precision of the layers' fake quantisation
-    to apply to the operand inside the generators (None: operand as given)."""
-    _require_cuda(x, w)
-    if x.dim() != 4 or w.dim() != 4 or x.size(1) != w.size(1):
+def _conv_desc(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config, xnor,
+               act_fake_quant, weight_fake_quant):
+    """(descriptor, channels-last flags) of a conv call; x may be a tensor or a (shape, channels_last) pair."""
+    if isinstance(x, torch.Tensor):
+        if x.dim() != 4:
+            raise RuntimeError("conv2d: expected input [N,C,H,W], got %s" % (tuple(x.shape),))
+        xshape, cl_a = tuple(x.shape), is_channels_last(x)
+    else:
+        xshape, cl_a = tuple(x[0]), bool(x[1])
+    if len(xshape) != 4 or w.dim() != 4 or xshape[1] != w.size(1):
         raise RuntimeError("conv2d: expected input [N,C,H,W] and weight [O,C,KH,KW] with equal C, got %s and %s"
-                           % (tuple(x.shape), tuple(w.shape)))
-    cl_a, cl_w = is_channels_last(x), is_channels_last(w)
-    xc, wc = _as_layout(x, cl_a), _as_layout(w, cl_w)
-    N, C, H, W = xc.shape
-    O, _, KH, KW = wc.shape
+                           % (xshape, tuple(w.shape)))
+    cl_w = is_channels_last(w)
+    N, C, H, W = xshape
+    O, _, KH, KW = w.shape
     fq = lambda p: 0 if p is None else int(p) + 1
     d = _lib.ConvDesc(N, C, H, W, O, KH, KW, int(padding[1]), int(padding[0]), int(stride[0]), int(stride[1]),
                       int(bit_length), int(lfsr_length), int(gen_config), int(bin_config),
                       int(prog_load[0]), int(prog_load[1]), int(prog_load[2]), int(cl_a), int(cl_w), int(bool(xnor)),
                       fq(act_fake_quant), fq(weight_fake_quant))
+    return d, cl_a, cl_w
+
+
+class PreparedWeightStreams:
+    """Weight bitstreams generated ahead of the conv call they belong to (sc_conv2d_prepare_weights)."""
+
+    def __init__(self, buf, key):
+        self.buf, self.key = buf, key
+
+
+def sc_conv2d_prepare_weights(x_like, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
+                              xnor=False, act_fake_quant=None, weight_fake_quant=None, into=None, keep_weight_copy=False):
+    """Generates the weight bitstreams of the conv call  sc_conv2d(x, w, <same arguments>, prepared=<result>)  on the
+    current stream, ahead of that call: a layer's weight streams depend on its weights alone, so they can be made on a
+    second stream while the previous layer computes.  x_like: the activation tensor or ((N, C, H, W), channels_last).
+    into: a PreparedWeightStreams of an earlier call with the same arguments, whose buffer is then reused.
+    keep_weight_copy: also store the copy of w that a WeightStreamCache compares with (not needed for prepared=)."""
+    _require_cuda(w)
+    d, _, cl_w = _conv_desc(x_like, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config, xnor,
+                            act_fake_quant, weight_fake_quant)
+    wc = _as_layout(w, cl_w)
     L = _lib.lib()
-    extended = want_value or weight_cache is not None
+    with torch.cuda.device(w.device):
+        nbytes = L.rexsc_conv2d_weight_streams_bytes(ctypes.byref(d))
+        if nbytes == 0:
+            _lib.check(-1, "rexsc_conv2d (planning)")
+        key = d.key()
+        if into is not None and into.key == key and into.buf.numel() >= nbytes and into.buf.device == w.device:
+            buf = into.buf
+        else:
+            buf = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+        rc = L.rexsc_conv2d_prepare_weights(ctypes.byref(d), _ptr(wc), _ptr(buf), buf.numel(), int(bool(keep_weight_copy)),
+                                            _stream())
+        _lib.check(rc, "rexsc_conv2d_prepare_weights")
+    return PreparedWeightStreams(buf, key)
+
+
+def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config,
+              want_split=True, want_diff=False, xnor=False, want_value=False, weight_cache=None,
+              act_fake_quant=None, weight_fake_quant=None, prepared=None):
+    """SC conv2d on the HIP path.  padding=(p0,p1): p0 pads the LAST axis, p1 axis 2, as the
+    reference's F::pad call does (sc_conv.cpp:314); stride=(s0,s1): s0 along axis 2.
+    -> (pos, neg, diff) int16, plus the float32 tensor pos / L - neg / L as a fourth element when want_value.
+    weight_cache: a WeightStreamCache that keeps w's bitstreams between calls (the device checks on every call that
+    they still belong to w's values).  act_fake_quant / weight_fake_quant: precision of the layers' fake quantisation
+    to apply to the operand inside the generators (None: operand as given).  prepared: the weight streams of exactly
+    this call, made by sc_conv2d_prepare_weights on a stream this one is ordered after (the caller's word: no check)."""
+    _require_cuda(x, w)
+    d, cl_a, cl_w = _conv_desc(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_config, gen_config, xnor,
+                               act_fake_quant, weight_fake_quant)
+    xc, wc = _as_layout(x, cl_a), _as_layout(w, cl_w)
+    N, C, H, W = xc.shape
+    O, _, KH, KW = wc.shape
+    L = _lib.lib()
+    extended = want_value or weight_cache is not None or prepared is not None
     with torch.cuda.device(x.device):
         Ho = (H + 2 * d.pad_h - KH) // d.stride_h + 1
         Wo = (W + 2 * d.pad_w - KW) // d.stride_w + 1
@@ -163,7 +214,11 @@ def sc_conv2d(x, w, bit_length, lfsr_length, padding, stride, prog_load, bin_con
             return pos, neg, diff
         value = mk(want_value, torch.float32)
         wbuf, mode = None, _lib.WSTREAMS_FILL
-        if weight_cache is not None:
+        if prepared is not None:
+            if prepared.key != d.key():
+                raise RuntimeError("conv2d: the prepared weight streams belong to another call (descriptor differs)")
+            wbuf, mode = prepared.buf, _lib.WSTREAMS_TRUST
+        elif weight_cache is not None:
             wbuf, mode = weight_cache.lookup(("conv",) + d.key(), L.rexsc_conv2d_weight_streams_bytes(ctypes.byref(d)),
                                              x.device)
         rc = L.rexsc_conv2d_orn_ex(ctypes.byref(d), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(diff), _ptr(value),

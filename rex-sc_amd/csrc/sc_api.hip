@@ -362,6 +362,27 @@ int kept_weights_changed(const ScPlan &pl, const float *w, void *wstreams, int m
                             mode == REXSC_WSTREAMS_FILL, stream);
 }
 
+// Weight streams (and the activation generator's table, and the folded streams) of a conv plan.  wstreams != nullptr: a
+// kept buffer in mode REXSC_WSTREAMS_FILL or _VERIFY; nullptr: plain generation into the workspace.
+int generate_weight_streams(const ScPlan &pl, int C, const float *w, uint32_t *Wst, uint32_t *tab_a, uint32_t *W2,
+                            void *wstreams, int mode, hipStream_t stream)
+{
+    const unsigned long long *guard = nullptr;
+    unsigned long long epoch = 0;
+    int rc;
+    if (wstreams) {
+        rc = kept_weights_changed(pl, w, wstreams, mode, &guard, &epoch, stream);
+        if (rc) return rc;
+    }
+    rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream, guard, epoch);
+    if (rc) return rc;
+    if (pl.fold) {
+        rc = fold_weight_streams(Wst, W2, pl.cp.n_slots, pl.fold_KH, pl.fold_KW, pl.wg.O_pad, C, stream, guard, epoch);
+        if (rc) return rc;
+    }
+    return REXSC_OK;
+}
+
 // The conv op proper: generators, compute, finalize, batch chunk by batch chunk, in `workspace`
 // (device memory of at least pl.total bytes).  wstreams != nullptr: the weight streams and the activation
 // generator's state-plane table live there (pl.wstream_total bytes) instead of in the workspace;
@@ -384,18 +405,8 @@ int run_conv(const ScPlan &pl, const rexsc_conv_desc *d, const float *x, const f
     }
     int rc;
     if (!wstreams || wstreams_valid != REXSC_WSTREAMS_TRUST) {
-        const unsigned long long *guard = nullptr;
-        unsigned long long epoch = 0;
-        if (wstreams) {
-            rc = kept_weights_changed(pl, w, wstreams, wstreams_valid, &guard, &epoch, stream);
-            if (rc) return rc;
-        }
-        rc = sng_weights(w, Wst, pl.wg, pl.gen_w, tab_a, &pl.ag, &pl.gen_act, stream, guard, epoch);
+        rc = generate_weight_streams(pl, d->C, w, Wst, tab_a, W2, wstreams, wstreams_valid, stream);
         if (rc) return rc;
-        if (pl.fold) {
-            rc = fold_weight_streams(Wst, W2, pl.cp.n_slots, pl.fold_KH, pl.fold_KW, pl.wg.O_pad, d->C, stream, guard, epoch);
-            if (rc) return rc;
-        }
     }
     const size_t in_image = (size_t)d->C * d->H * d->W;
     const size_t out_image = (size_t)d->O * pl.Ho * pl.Wo;
@@ -516,6 +527,30 @@ extern "C" int rexsc_conv2d_orn_ex(const rexsc_conv_desc *d, const float *x, con
         return REXSC_ERR_WORKSPACE;
     }
     return run_conv(pl, d, x, w, out_pos, out_neg, out_diff, out_value, weight_streams, weight_streams_valid, workspace, stream);
+}
+
+// The weight half of rexsc_conv2d_orn_ex on its own: fills the kept buffer as a call in mode REXSC_WSTREAMS_FILL would
+// (keep_weight_copy = 0: without the copy of the weights that a later VERIFY compares with), so that the conv call proper
+// can follow in mode TRUST (or VERIFY).  The weight streams of a layer depend on nothing but its weights: a caller can
+// issue this on another stream while the previous layer computes.
+extern "C" int rexsc_conv2d_prepare_weights(const rexsc_conv_desc *d, const float *w, void *weight_streams,
+                                            size_t weight_streams_bytes, int keep_weight_copy, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    ScPlan pl;
+    int rc = plan_conv(pl, d);
+    if (rc) return rc;
+    REXSC_CHECK_ARG(w && weight_streams, "null pointer");
+    if (weight_streams_bytes < pl.wstream_total) {
+        set_error("conv2d: weight-stream buffer of %zu bytes needed, %zu given", pl.wstream_total, weight_streams_bytes);
+        return REXSC_ERR_WORKSPACE;
+    }
+    uint8_t *base = (uint8_t *)weight_streams;
+    uint32_t *tab_a = pl.tab_a_words ? (uint32_t *)(base + pl.wstream_off_tab) : nullptr;
+    uint32_t *W2 = pl.fold ? (uint32_t *)(base + pl.wstream_off_w2) : nullptr;
+    // without the copy of the weights the buffer cannot be verified later: plain generation into it
+    return generate_weight_streams(pl, d->C, w, (uint32_t *)weight_streams, tab_a, W2, keep_weight_copy ? weight_streams : nullptr,
+                                   REXSC_WSTREAMS_FILL, stream);
 }
 
 // Same op with the workspace taken from the library's static device array: no allocation of any kind,

@@ -122,6 +122,38 @@ def test_kept_weight_streams_are_used_until_the_weights_change():
     assert torch.equal(_ops.sc_conv2d(*args, weight_cache=cache)[0], want2[0])
 
 
+@pytest.mark.parametrize("cfg", [(2, 128, 14, 14, 64, 3, 1, 32, 1, True), (4, 3, 16, 16, 32, 3, 1, 64, 2, False)],
+                         ids=["c128", "c3_folded_taps"])
+def test_weight_streams_prepared_ahead_on_a_second_stream(cfg):
+    """rexsc_conv2d_prepare_weights on a side stream, the conv call proper on the caller's stream after an event:
+    same results as the one-call form; the buffer is reused for new weight values; a buffer made for another
+    descriptor is refused."""
+    import _ops
+    x, w, xt, wt = _operands(cfg, seed=21)
+    N, C, H, W, O, K, stride, L, bc, cla = cfg
+    args = (L, -1, (K // 2, K // 2), (stride, stride), (7, 8, 1), bc, 1)
+    want = _ops.sc_conv2d(xt, wt, *args)
+    side = torch.cuda.Stream()
+    cur = torch.cuda.current_stream()
+    prepared = None
+    for rnd in range(3):
+        if rnd == 2:
+            wt.data.mul_(-0.5)
+            want = _ops.sc_conv2d(xt, wt, *args)
+        side.wait_stream(cur)
+        with torch.cuda.stream(side):
+            prepared = _ops.sc_conv2d_prepare_weights(((N, C, H, W), cla), wt, *args, into=prepared)
+            ev = torch.cuda.Event()
+            ev.record(side)
+        cur.wait_event(ev)
+        got = _ops.sc_conv2d(xt, wt, *args, prepared=prepared)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]) and int(want[0].max()) > 0
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="another call"):
+        _ops.sc_conv2d(xt[:1].contiguous(memory_format=torch.channels_last if cla else torch.contiguous_format), wt, *args,
+                       prepared=prepared)
+
+
 def _oracle_layer_value(x, w, prec, L, padding, stride, cla):
     xq, wq = orc.quantize(x.cpu().numpy(), prec), orc.quantize(w.cpu().numpy(), prec)
     opos, oneg = orc.conv2d_generic_general_split(xq, wq, L, -1, 16, padding, stride, (7, 8, 1), 1, 1,
