@@ -199,6 +199,20 @@ def main():
         "roofline": roofline,
     }
 
+    # the same step with the stream generators of the reference's CUDA kernels (REXSC_XNOR_MODE=cuda_ref: other
+    # sequence tables and seed offsets, the same kernels)
+    prev_mode = os.environ.get("REXSC_XNOR_MODE")
+    os.environ["REXSC_XNOR_MODE"] = "cuda_ref"
+    try:
+        sec_xnor = time_gpu(torch, step, max(3, args.steps // 2), 2)
+        out["config"]["xnor_mode_cuda_ref"] = {"ms_per_step": sec_xnor * 1e3, "bit_mac_per_s": total_mac * L / sec_xnor,
+                                               "relative_to_headline": sec_xnor / sec}
+    finally:
+        if prev_mode is None:
+            os.environ.pop("REXSC_XNOR_MODE", None)
+        else:
+            os.environ["REXSC_XNOR_MODE"] = prev_mode
+
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_sample_batch, L, OR_N, full_batch=N)
     if not args.no_extra:
@@ -304,7 +318,7 @@ def cpu_baseline(sample_batch, L, or_n, full_batch=64):
 def cpu_baselines_other_configs(torch):
     """The C restatement in oracle/ (kind "port", OpenMP) on the tensors bench_extra.py builds for configurations 1, 2
     and 4 (same seeds, same generator calls): configurations 1 and 2 at full size, the fixed-point conv on the first two
-    images of each shape."""
+    images of each shape; configuration 3: its four SC conv layers at full batch on synthetic operands."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle as orc
     cores = orc.num_threads()
@@ -325,6 +339,20 @@ def cpu_baselines_other_configs(torch):
     sec = time.perf_counter() - t0
     res["config2_sc_linear"] = {"value": 256 * 4096 * 1024 * 64 / sec, "unit": "bit-MAC/s", "cores": cores, "kind": "port",
                                 "sample": "the same tensors at full size (%.2f s)" % sec}
+    # configuration 3: the four SC conv layers of the TinyConv net (OR-3, 64-bit streams) at its batch of 256, on
+    # synthetic operands of the layers' shapes (the net's own activations exist only inside its forward pass)
+    g = torch.Generator().manual_seed(3)
+    sec = 0.0
+    for C, H, O in ((3, 32, 32), (32, 32, 32), (32, 16, 64), (64, 16, 64)):
+        x = (torch.randint(0, 64, (256, C, H, H), generator=g).float() / 64).numpy()
+        w = ((torch.randn(O, C, 3, 3, generator=g) * (2.0 / (O * 9)) ** 0.5) * 64).round().clamp(-63, 63).div(64).numpy()
+        t0 = time.perf_counter()
+        orc.conv2d_generic_general_split(x, w, 64, -1, 16, (1, 1), (1, 1), (7, 8, 1), 2, 1)
+        sec += time.perf_counter() - t0
+    res["config3_tinyconv_train"] = {
+        "value": 256 / sec, "unit": "images/s", "cores": cores, "kind": "port",
+        "sample": "the SC forward of the net's four SC conv layers alone (3-32-32 at 32x32, 32-64-64 at 16x16; OR-3, "
+                  "64-bit streams), batch 256, synthetic operands of the layers' shapes (%.2f s)" % sec}
     for C, H in ((64, 56), (128, 28), (256, 14), (512, 7)):
         g = torch.Generator().manual_seed(4)
         x = (torch.randint(0, 32, (64, C, H, H), generator=g).float() / 32)[:2].numpy()

@@ -40,6 +40,21 @@ def build_oracle(force=True):
     return ORACLE_SO
 
 
+ORACLE_SAN_SO = os.path.join(os.path.dirname(ORACLE_SO), "librexsc_oracle_san.so")
+
+
+def build_oracle_sanitized():
+    """The same source with AddressSanitizer and UndefinedBehaviorSanitizer (host code only; any finding aborts).
+    -> (library path, path of the ASan runtime that a process loading it has to preload)."""
+    os.makedirs(os.path.dirname(ORACLE_SAN_SO), exist_ok=True)
+    src = os.path.join(HERE, "rexsc_oracle.c")
+    _run(["gcc", "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
+          "-fno-sanitize-recover=undefined", "-march=x86-64-v3", "-fopenmp", "-fPIC", "-shared", "-std=gnu11",
+          "-Wall", "-o", ORACLE_SAN_SO, src, "-lm"])
+    runtime = subprocess.run(["gcc", "-print-file-name=libasan.so"], capture_output=True, text=True).stdout.strip()
+    return ORACLE_SAN_SO, runtime
+
+
 def ref_available():
     return os.path.isdir(REF_SRC)
 

@@ -28,7 +28,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "_build", "librexsc_oracle.so")
+# REXSC_ORACLE_SO: another build of the same source (the sanitizer build of tests/test_oracle_sanitizers.py)
+_SO = os.environ.get("REXSC_ORACLE_SO") or os.path.join(_HERE, "_build", "librexsc_oracle.so")
 _lib = None
 
 _i32p = ctypes.POINTER(ctypes.c_int32)

@@ -372,7 +372,9 @@ static inline int orc_saturate_shift(int value, int max_value, int d)
 {   /* fixed.cpp:56-60 */
     int vs = value < max_value ? value : max_value;
     int round_bit = (vs >> (d - 1 > 0 ? d - 1 : 0)) % 2;
-    return ((vs >> d) + round_bit) << d;
+    /* The OR adders can hand a negative sum in.  The reference shifts it left as it is (what its compiler makes of
+     * that is a multiplication by 2^d); written as the multiplication here, which is defined for negative values. */
+    return ((vs >> d) + round_bit) * (1 << d);
 }
 
 typedef struct { int v1, v2; } orc_or2_t;
