@@ -173,10 +173,12 @@ int rexsc_linear_orn_ex(const rexsc_linear_desc *d, const float *x, const float 
  * utils_class.py:183-208) on the same kernels: operands q = ceil(float16(x * L)) with activations
  * unclamped and weight parts clamped to weight_clamp (the function's `prec - 1`: 127), seeds
  * (67 + c) % P + 1 / (37 + c) % P + 1 for the positive / negative weight part and c % P + 1 for
- * activations, P = L - 1.  bin_config 0 is its forward 'full_or' (per-cycle OR), 51200 its 'full_bin'.
+ * activations, P = L - 1; share = 0 is the function's share=False: one generator per element, the index c replaced
+ * by the element's index in the whole tensor (o * C + c for weights, b * C + c for activations; :996-998).
+ * bin_config 0 is its forward 'full_or' (per-cycle OR), 51200 its 'full_bin'.
  * bit_length 8..128, lfsr_length <= 0, gen_config 1, no progressive loading.  Outputs are the per-output
  * sums over the L cycles (the function returns them divided by L).  Workspace: rexsc_linear_workspace_bytes. */
-int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp, const float *x, const float *w,
+int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp, int share, const float *x, const float *w,
                         int32_t *out_pos, int32_t *out_neg,
                         void *workspace, size_t workspace_bytes, rexsc_stream_t stream);
 

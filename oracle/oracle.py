@@ -289,7 +289,7 @@ def compute_bias_std_coef(or_n, a_bit, a_act, order):
     return bias_coef, std_coef
 
 
-def linear_generic_legacy(x, w, bit_length, forward="full_or", prec=128):
+def linear_generic_legacy(x, w, bit_length, forward="full_or", prec=128, share=True):
     """The reference's legacy `linear_generic` (utils_functional.py:955-1081; generator 'lfsr', share=True) with
     its generators (:147-165 lfsr_init, :254-272 lfsr_cont) -> float32 [B,O], pos - neg.
 
@@ -297,8 +297,9 @@ def linear_generic_legacy(x, w, bit_length, forward="full_or", prec=128):
     prec-1 per polarity, activations unclamped; :980-995), LFSR states are integers stepped before the compare
     (:1022), seeds c % P + 1 / (67 + c) % P + 1 / (37 + c) % P + 1 with P = L - 1 shared by all rows (:1000-1001),
     per cycle sign(count) ('full_or') or count ('full_bin') (:1031-1036), mean over cycles rounded to float16
-    (compute_type, :28; :1067-1068).  Pinned by tests/golden/ref_linear_legacy.npz, written by the reference's own
-    function."""
+    (compute_type, :28; :1067-1068).  share=False (:996-998): one generator per element, the seed index running over
+    the whole weight tensor (o * C + c) and the whole activation tensor (b * C + c).  Pinned by
+    tests/golden/ref_linear_legacy.npz, written by the reference's own function."""
     x = np.asarray(x, np.float32)
     w = np.asarray(w, np.float32)
     L = int(bit_length)
@@ -310,8 +311,12 @@ def linear_generic_legacy(x, w, bit_length, forward="full_or", prec=128):
     wp = np.clip(w * Lf, 0, bit_range).astype(np.float16).astype(np.float32)
     wn = (-np.clip(w * Lf, -bit_range, 0)).astype(np.float16).astype(np.float32)
     C = x.shape[1]
-    c = np.arange(C)
-    st_a, st_p, st_n = c % P + 1, (67 + c) % P + 1, (37 + c) % P + 1
+    if share:
+        c = np.arange(C)
+        st_a, st_p, st_n = c % P + 1, (67 + c) % P + 1, (37 + c) % P + 1
+    else:
+        ia, iw = np.arange(x.size).reshape(x.shape), np.arange(w.size).reshape(w.shape)
+        st_a, st_p, st_n = ia % P + 1, (67 + iw) % P + 1, (37 + iw) % P + 1
     step = np.vectorize(lambda v: lfsr_step(lb, 0, int(v)))
     pos = np.zeros((x.shape[0], w.shape[0]), np.float64)
     neg = np.zeros_like(pos)

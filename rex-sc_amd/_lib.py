@@ -71,7 +71,7 @@ SIGNATURES = {
     "rexsc_linear_orn": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "rexsc_linear_weight_streams_bytes": (_sz, [ctypes.POINTER(LinearDesc)]),
     "rexsc_linear_orn_ex": (_int, [ctypes.POINTER(LinearDesc), _vp, _vp, _vp, _vp, _vp, _sz, _int, _vp, _sz, _vp]),
-    "rexsc_linear_legacy": (_int, [ctypes.POINTER(LinearDesc), _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "rexsc_linear_legacy": (_int, [ctypes.POINTER(LinearDesc), _int, _int, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "rexsc_orn_forward": (_int, [_vp, _vp, _sz, _int, _vp]),
     "rexsc_orn_backward": (_int, [_vp, _vp, _vp, _sz, _int, _int, _vp]),
     "rexsc_orn_bias_std_both_forward": (_int, [_vp, _vp, _vp, _vp, _vp, _sz, _int, _u64, _u64, _vp, _vp, _vp, _vp]),

@@ -271,9 +271,10 @@ def sc_linear(x, w, prog_load, bit_length, lfsr_length, bin_config, gen_config, 
     return pos, neg
 
 
-def sc_linear_legacy(x, w, bit_length, bin_config, weight_clamp=127):
+def sc_linear_legacy(x, w, bit_length, bin_config, weight_clamp=127, share=True):
     """The reference's legacy `linear_generic` simulation (utils_functional.py:955-1081, generator 'lfsr',
-    shared generators) on the HIP kernels -> (pos, neg) int32 [B,O]: per-output sums over the bit_length cycles."""
+    shared generators, or one per element with share=False) on the HIP kernels -> (pos, neg) int32 [B,O]: per-output
+    sums over the bit_length cycles."""
     _require_cuda(x, w)
     if x.dim() != 2 or w.dim() != 2 or x.size(1) != w.size(1):
         raise RuntimeError("linear: expected input [B,C] and weight [O,C], got %s and %s"
@@ -294,7 +295,7 @@ def sc_linear_legacy(x, w, bit_length, bin_config, weight_clamp=127):
         pos = torch.empty((B, O), dtype=torch.int32, device=x.device)
         neg = torch.empty((B, O), dtype=torch.int32, device=x.device)
         ws = _workspace(ws_bytes, x.device)
-        rc = L.rexsc_linear_legacy(ctypes.byref(d), int(weight_clamp), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws),
+        rc = L.rexsc_linear_legacy(ctypes.byref(d), int(weight_clamp), int(bool(share)), _ptr(xc), _ptr(wc), _ptr(pos), _ptr(neg), _ptr(ws),
                                    ws.numel(), _stream())
         _lib.check(rc, "rexsc_linear_legacy")
     return pos, neg

@@ -228,8 +228,8 @@ __device__ __forceinline__ void fixed_pack_w16(const float *__restrict__ w, int8
     }
 }
 
-// One launch prepares everything the MFMA kernel needs: blocks [0, act_blocks) pack the activations,
-// the next w_blocks pack the weights, the last zero_blocks clear the output when the reduction is split
+// One launch prepares everything the MFMA kernel needs: the first w_blocks blocks pack the weights, the next
+// act_blocks pack the activations, the last zero_blocks clear the output when the reduction is split
 // over blocks that add their parts atomically.  (Three launches of this size cost more in launch
 // latency than in work.)
 __global__ __launch_bounds__(256) void fixed_prepare_kernel(const float *__restrict__ x, int8_t *__restrict__ xq16,
@@ -238,11 +238,13 @@ __global__ __launch_bounds__(256) void fixed_prepare_kernel(const float *__restr
                                                             size_t n_out, Fixed8Params p, unsigned act_blocks,
                                                             unsigned w_blocks, unsigned zero_blocks)
 {
+    // the few weight blocks come first in the grid: their strided loads then run beside the activation blocks
+    // instead of forming a round of their own at the end of the launch
     unsigned bid = blockIdx.x;
-    if (bid < act_blocks) { fixed_pack_act16(x, xq16, p, bid); return; }
-    bid -= act_blocks;
     if (bid < w_blocks) { fixed_pack_w16(w, wq16, wp16, p, bid, w_blocks); return; }
     bid -= w_blocks;
+    if (bid < act_blocks) { fixed_pack_act16(x, xq16, p, bid); return; }
+    bid -= act_blocks;
     if ((reinterpret_cast<uintptr_t>(out) & 15) == 0) {
         uint4 *o4 = reinterpret_cast<uint4 *>(out);
         const size_t n4 = n_out / 4;

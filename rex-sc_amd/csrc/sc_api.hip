@@ -667,9 +667,10 @@ extern "C" int rexsc_linear_orn_ex(const rexsc_linear_desc *d, const float *x, c
 //     clamped to weight_clamp (the function's `prec - 1`, 127 by default) -- the simulation compares the
 //     float16 products with integer LFSR states, and v > s for an integer s is ceil(v) > s;
 //   * seeds (67 + c) % P + 1 for the positive and (37 + c) % P + 1 for the negative weight part, c % P + 1
-//     for activations (utils_functional.py:147-165).
+//     for activations (utils_functional.py:147-165); share == 0: the function's share=False, where c is replaced by
+//     the element's index in the whole tensor (o * C + c, b * C + c).
 // Two passes over one set of activation streams, one per weight polarity (each with its own seeds).
-extern "C" int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp, const float *x, const float *w,
+extern "C" int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp, int share, const float *x, const float *w,
                                    int32_t *out_pos, int32_t *out_neg, void *workspace, size_t workspace_bytes,
                                    rexsc_stream_t stream_)
 {
@@ -695,6 +696,14 @@ extern "C" int rexsc_linear_legacy(const rexsc_linear_desc *d, int weight_clamp,
     const float L = (float)d->bit_length;
     pl.gen_act.legacy = 1; pl.gen_act.clamp_hi = L;
     pl.gen_w.legacy = 1; pl.gen_w.clamp_hi = weight_clamp < d->bit_length ? (float)weight_clamp : L;
+    if (!share) {
+        // one generator per element (utils_functional.py:996-998): the seed index runs over the whole weight tensor
+        // (o * C + c) and the whole activation tensor (b * C + c).  The activation generator's table was planned for
+        // seeds that do not depend on the row: the lane-ballot generator takes over.
+        pl.wg.seed_omul = d->C;
+        pl.ag.seed_pmul = d->C;
+        tab_a = nullptr;
+    }
     for (int pol = 0; pol < 2; pol++) {
         pl.gen_w.seed_add = pol == 0 ? 67 : 37;
         pl.gen_w.sign = pol == 0 ? 1.f : -1.f; // pass 1 streams -w: its positive part is w's negative part

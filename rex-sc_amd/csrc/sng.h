@@ -21,6 +21,9 @@ struct WeightGeom {
     int O, C, KH, KW;
     int channels_last;
     int ZC, ZG, O_pad;
+    // seed index += o * seed_omul.  0 everywhere but in the reference's legacy linear simulation with one generator
+    // per weight (utils_functional.py:996-998), where the index runs over the whole tensor: o * C + c.
+    int seed_omul;
 };
 
 // Words of LFSR state-plane table the bit-sliced activation generator needs for this problem, or 0

@@ -689,7 +689,8 @@ __global__ __launch_bounds__(256) void sng_weight_kernel(const float *__restrict
                     const int combo = combo0 + cl;
                     const int h = combo % HALVES, kx = combo / HALVES;
                     const long c = (long)zg * CCH + h * 64 + lane;
-                    const int sd = (int)(((long)gp.seed_add + c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
+                    // (+ o * seed_omul for generators that differ per output channel: blocks then hold one channel each)
+                    const int sd = (int)(((long)gp.seed_add + (long)og * wog * geo.seed_omul + c * geo.KH * KW + ky * KW + kx) % gp.seed_mod);
                     s_pos[cl * 64 + lane] = s_inv[sd + gp.seed_off];
                 }
                 __syncthreads();
@@ -853,6 +854,7 @@ static int launch_weight(const float *w, uint32_t *Wst, const SeqTable *tables, 
     const char *tune = getenv("REXSC_TUNE_WSNG_BLOCKS");
     const long min_blocks = tune && atoi(tune) > 0 ? atoi(tune) : 768;
     while (wog > 2 && (long)(geo.O_pad / wog) * geo.KH * geo.ZG < min_blocks) wog /= 2;
+    if (geo.seed_omul) wog = 1; // the state planes a block computes once serve one output channel only
     const long n_wblocks = (long)(geo.O_pad / wog) * geo.KH * geo.ZG;
     REXSC_CHECK_ARG(n_wblocks < (1L << 31), "weight SNG: grid too large");
     if (job.T) {

@@ -626,8 +626,10 @@ def linear_generic(activation, weight, **kwargs):
     numbers from the HIP kernels here (rexsc_linear_legacy).
 
     bit_length, prec (128), share (True), generator, forward ('full_or' | 'full_bin') mean what they mean in the
-    reference.  Live configuration only: generator 'lfsr' with shared generators; the simulated true-random
-    generator, 'lfsr_split' and share=False are not built and raise.  The forward value is the SC result
+    reference.  generator 'lfsr' with share=True (one generator per input feature) or share=False (one per weight and
+    per activation element, :996-998) is built.  The other two generators have no result to reproduce: 'lfsr_split'
+    draws its main streams from torch.randint on every cycle (the test at :1017 sends every generator but 'lfsr' to
+    rand_init) and the "true random" generator is torch.randint by design; they raise.  The forward value is the SC result
     (sum over the cycles / bit_length, the simulation's `.mean(0)`), gradients are those of the float surrogate
     1 - exp(-x w_pos^T) - (1 - exp(-x w_neg^T)) ('full_or') or x w^T ('full_bin').  The reference's result tensor
     ends up float16 (its compute_type, :28-29); the values here are the same numbers as float32 -- for 'full_bin'
@@ -639,9 +641,9 @@ def linear_generic(activation, weight, **kwargs):
     forward = setvalue_default(kwargs, "forward", "full_or")
     if forward not in ("full_or", "full_bin"):
         raise ValueError("linear_generic: forward must be 'full_or' or 'full_bin' (got %r)" % (forward,))
-    if generator != "lfsr" or not share:
-        raise ValueError("linear_generic: only generator='lfsr' with share=True is built (got generator=%r, share=%r)"
-                         % (generator, share))
+    if generator != "lfsr":
+        raise ValueError("linear_generic: only generator='lfsr' is built; the reference's other generators draw from "
+                         "torch.randint and have no reproducible result (got generator=%r)" % (generator,))
     bit_range = prec - 1  # taken before prec follows the stream length (:973, :980-981)
     w_pos = weight.clamp(0, 100)
     w_neg = -(weight.clamp(-100, 0))
@@ -655,7 +657,7 @@ def linear_generic(activation, weight, **kwargs):
     if os.environ.get("Global_Sync", "1") == "1":
         with torch.no_grad():
             pos, neg = _ops.sc_linear_legacy(activation.data, weight.data, bit_length, 0 if forward == "full_or" else 51200,
-                                             weight_clamp=bit_range)
+                                             weight_clamp=bit_range, share=bool(share))
             mean = lambda t: (t.to(torch.float32) / bit_length).to(torch.float16).to(result_pos_value.dtype)
             result_pos_value.data = mean(pos)
             result_neg_value.data = mean(neg)

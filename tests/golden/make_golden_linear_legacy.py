@@ -37,6 +37,11 @@ CASES = [
     ("bin_L32_q7", 5, 70, 7, 32, "full_bin", "q7", 0.5),
     ("bin_L128_plain", 4, 200, 5, 128, "full_bin", "plain", 0.7),
     ("or_L128_dense_ones", 3, 40, 4, 128, "full_or", "ones", 0.25),  # activations of exactly 1.0, weights of +-1.0
+    # share=False: one generator per weight and per activation element, seeds running over the whole tensors (:996-998)
+    ("or_L32_q7_noshare", 5, 64, 8, 32, "full_or", "q7", 0.25, False),
+    ("or_L128_q7_noshare", 6, 100, 9, 128, "full_or", "q7", 0.2, False),
+    ("bin_L64_plain_noshare", 4, 70, 17, 64, "full_bin", "plain", 0.5, False),   # 17 outputs: a ragged group of 16
+    ("or_L16_q7_noshare", 3, 33, 5, 16, "full_or", "q7", 0.3, False),
 ]
 
 
@@ -58,12 +63,14 @@ def operands(rng, kind, B, C, O, dens):
 def main():
     rng = np.random.default_rng(6737)
     out, meta = {}, []
-    for (name, B, C, O, L, forward, kind, dens) in CASES:
+    for case in CASES:
+        (name, B, C, O, L, forward, kind, dens), share = case[:8], (case[8] if len(case) > 8 else True)
         x, w = operands(rng, kind, B, C, O, dens)
-        y = ref.linear_generic(torch.from_numpy(x), torch.from_numpy(w), bit_length=L, forward=forward, generator="lfsr")
+        y = ref.linear_generic(torch.from_numpy(x), torch.from_numpy(w), bit_length=L, forward=forward, generator="lfsr",
+                               share=share)
         y = y.detach().float().numpy()
         out[name + "/x"], out[name + "/w"], out[name + "/y"] = x, w, y
-        meta.append(dict(name=name, bit_length=L, forward=forward))
+        meta.append(dict(name=name, bit_length=L, forward=forward, share=share))
         print(name, "out", y.shape, "min %.4f max %.4f nonzero %.2f" % (y.min(), y.max(), (y != 0).mean()))
     out["meta"] = np.frombuffer(json.dumps(meta).encode(), dtype=np.uint8)
     path = os.path.join(HERE, "ref_linear_legacy.npz")

@@ -26,7 +26,8 @@ def test_legacy_linear_golden(case, sng_mode, monkeypatch):
     n = case["name"]
     print("legacy linear golden", n, "sng mode", sng_mode, flush=True)
     x, w = torch.from_numpy(_g[n + "/x"]).cuda(), torch.from_numpy(_g[n + "/w"]).cuda()
-    y = uf.linear_generic(x, w, bit_length=case["bit_length"], forward=case["forward"], generator="lfsr")
+    y = uf.linear_generic(x, w, bit_length=case["bit_length"], forward=case["forward"], generator="lfsr",
+                          share=case.get("share", True))
     assert y.dtype == torch.float32
     assert np.array_equal(y.cpu().numpy(), _g[n + "/y"])
 
@@ -39,13 +40,16 @@ SHAPES = [
     (16, 300, 24, 16, "full_bin", "plain"),
     (8, 4096, 12, 128, "full_bin", "q7"),      # sums above 65535: wide accumulators
     (5, 37, 3, 8, "full_or", "q7"),
+    (40, 300, 50, 32, "full_or", "q7", False),     # share=False: one generator per element
+    (9, 1000, 33, 128, "full_bin", "plain", False),
 ]
 
 
 @pytest.mark.parametrize("cfg", SHAPES, ids=lambda c: "_".join(str(v) for v in c))
 def test_legacy_linear_vs_oracle(cfg):
     import _ops
-    B, C, O, L, forward, kind = cfg
+    B, C, O, L, forward, kind = cfg[:6]
+    share = cfg[6] if len(cfg) > 6 else True
     print("legacy linear", cfg, flush=True)
     rng = np.random.default_rng(hash(cfg) & 0xFFFF)
     dens = 1.0 if forward == "full_bin" else min(1.0, 12.0 / np.sqrt(C) / 4)
@@ -58,17 +62,17 @@ def test_legacy_linear_vs_oracle(cfg):
     x = (x * (rng.uniform(size=x.shape) < dens)).astype(np.float32)
     w = (w * (rng.uniform(size=w.shape) < dens)).astype(np.float32)
     pos, neg = _ops.sc_linear_legacy(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), L,
-                                     0 if forward == "full_or" else 51200)
+                                     0 if forward == "full_or" else 51200, share=share)
     assert pos.dtype == torch.int32
     mean = lambda t: (t.float() / L).half().float().cpu().numpy()
-    want = orc.linear_generic_legacy(x, w, L, forward)
+    want = orc.linear_generic_legacy(x, w, L, forward, share=share)
     assert np.abs(want).max() > 0
     assert np.array_equal(mean(pos) - mean(neg), want)
     if forward == "full_bin" and C >= 4096:
         assert int(pos.max()) > 65535
     # the positive sums do not depend on the negative weights and vice versa (separate passes, separate seeds)
     p2, _ = _ops.sc_linear_legacy(torch.from_numpy(x).cuda(), torch.from_numpy(np.maximum(w, 0)).cuda(), L,
-                                  0 if forward == "full_or" else 51200)
+                                  0 if forward == "full_or" else 51200, share=share)
     assert torch.equal(p2, pos)
 
 

@@ -110,6 +110,7 @@ def test_legacy_linear_generic_matches_reference_python(case):
     """oracle.linear_generic_legacy against the vectors written by the reference's own linear_generic."""
     g, _ = _legacy_linear_cases()
     n = case["name"]
-    got = orc.linear_generic_legacy(g[n + "/x"], g[n + "/w"], case["bit_length"], case["forward"])
+    got = orc.linear_generic_legacy(g[n + "/x"], g[n + "/w"], case["bit_length"], case["forward"],
+                                    share=case.get("share", True))
     assert np.abs(g[n + "/y"]).max() > 0
     assert np.array_equal(got, g[n + "/y"])
