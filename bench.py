@@ -22,6 +22,7 @@ The one JSON line printed at the end also carries
                 conv, pointwise kernels, training steps), each with its own rate.
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -59,14 +60,22 @@ def make_conv_operands(torch, N, C, H, O, K, L, seed, channels_last=True):
 
 
 def time_gpu(torch, fn, steps, warmup):
+    """Seconds per call: `warmup` untimed calls, then exactly `steps` calls between two device synchronisations
+    (Python's cyclic garbage collector held off meanwhile, as timeit does)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
+    gc_was_on = gc.isenabled()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+    finally:
+        if gc_was_on:
+            gc.enable()
 
 
 def main():

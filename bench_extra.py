@@ -13,6 +13,9 @@ pass separate from the wall-clock timing.  The streaming kernels are timed twice
 buffers, so that every byte comes from and goes to HBM; `hbm_frac` is the rotating figure.
 """
 import ctypes
+import gc
+import json
+import os
 import time
 
 # integer VALU roofs, lane-ops/s (see bench.py): and + popcount pair at 2 + 4 cycles per wave64 and SIMD; single
@@ -28,14 +31,22 @@ STREAM_KERNELS = ("orn_", "sc_counts_to_float", "quantize", "split_weight", "mer
 
 
 def _time(torch, fn, steps, warmup):
+    """Seconds per call of fn over `steps` calls after `warmup` untimed ones; Python's cyclic garbage collector is
+    held off during the timed calls, as timeit does (a full collection is tens of milliseconds in this process)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        fn()
-    torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
+    gc_was_on = gc.isenabled()
+    gc.disable()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+    finally:
+        if gc_was_on:
+            gc.enable()
 
 
 def _profile(torch, fn, reps):
@@ -142,18 +153,31 @@ def config2_sc_linear(torch, dev):
     return out
 
 
-def _train_flavours(torch, dev, net, make_batch, batch, steps, lr):
+def _train_flavours(torch, dev, net, make_batch, batch, steps, lr, only_autocast=False):
+    """Training steps as utils_own.py:96-171 runs them: sync 1 / 3 / 2 in float32; with only_autocast, sync 1 under
+    float16 autocast with a gradient scaler instead (the reference's `torch_type != torch.float32` branch,
+    :127-131,156-165)."""
     import torch.nn.functional as F
     opt = torch.optim.Adam(net.parameters(), lr=lr, weight_decay=1e-4)
+    scaler = torch.amp.GradScaler("cuda") if only_autocast else None
     out = {}
-    for name, sync, frac in (("sync1_sc_forward", 1, 1.0), ("sync3_error_injection", 3, 1.0),
-                             ("sync2_calibration_half_batch", 2, 0.5)):
+    flavours = ((("sync1_sc_forward_autocast_fp16", 1, 1.0),) if only_autocast else
+                (("sync1_sc_forward", 1, 1.0), ("sync3_error_injection", 3, 1.0), ("sync2_calibration_half_batch", 2, 0.5)))
+    for name, sync, frac in flavours:
         n = max(1, int(batch * frac))
         x, y = make_batch(n)
 
         def step():
             net.sync = sync
             opt.zero_grad(set_to_none=True)
+            if only_autocast:
+                with torch.autocast("cuda", dtype=torch.float16):
+                    output = net(x)
+                loss = F.cross_entropy(output, y, label_smoothing=0.1)
+                scaler.scale(loss).backward()
+                scaler.step(opt)
+                scaler.update()
+                return loss
             loss = F.cross_entropy(net(x), y, label_smoothing=0.1)
             loss.backward()
             opt.step()
@@ -169,7 +193,7 @@ def _train_flavours(torch, dev, net, make_batch, batch, steps, lr):
     return out
 
 
-def config3_tinyconv_step(torch, dev):
+def config3_tinyconv_step(torch, dev, only_autocast=False):
     from sc_models import TinyConvSC
     torch.manual_seed(3)
     net = TinyConvSC(forward="or_3", err=6).to(dev)
@@ -179,10 +203,14 @@ def config3_tinyconv_step(torch, dev):
         return (torch.randn(n, 3, 32, 32, generator=g).clamp(-1, 1).to(dev),
                 torch.randint(0, 10, (n,), generator=g).to(dev))
 
-    res = _train_flavours(torch, dev, net, make_batch, 256, 10, 8e-3)
+    res = _train_flavours(torch, dev, net, make_batch, 256, 10, 8e-3, only_autocast)
     res["workload"] = ("TinyConv-style training step, batch 256, 3x32x32, conv3x3 3-32-32-pool-64-64-pool-fc10, "
                        "OR-3, 64-bit streams, Adam")
     return res
+
+
+def config3_tinyconv_autocast_step(torch, dev):
+    return config3_tinyconv_step(torch, dev, only_autocast=True)
 
 
 def _rotating_sets(nbytes_per_set):
@@ -251,7 +279,11 @@ def config4_fixed_conv(torch, dev):
     return out
 
 
-def config5_resnet18_step(torch, dev, batch=64):
+def config5_resnet18_autocast_step(torch, dev):
+    return config5_resnet18_step(torch, dev, only_autocast=True)
+
+
+def config5_resnet18_step(torch, dev, batch=64, only_autocast=False):
     from sc_models import ResNet18SC
     torch.manual_seed(5)
     net = ResNet18SC(forward="or_2", err=5).to(dev).to(memory_format=torch.channels_last)
@@ -261,9 +293,11 @@ def config5_resnet18_step(torch, dev, batch=64):
         return (torch.randn(n, 3, 224, 224, generator=g).to(dev).contiguous(memory_format=torch.channels_last),
                 torch.randint(0, 1000, (n,), generator=g).to(dev))
 
-    res = _train_flavours(torch, dev, net, make_batch, batch, 5, 1e-3)
+    res = _train_flavours(torch, dev, net, make_batch, batch, 5, 1e-3, only_autocast)
     res["workload"] = ("ResNet-18 SC training step, batch %d, 3x224x224, channels_last, OR-2, 32-bit streams, "
                        "float stem/fc, Adam" % batch)
+    if only_autocast:
+        return res
     # evaluation: weights frozen, the layers reuse their weight streams from call to call
     net.eval()
     net.sync = 1
@@ -368,6 +402,21 @@ def pointwise(torch, dev):
     return res
 
 
+def _in_child_process(name, timeout=240):
+    """One function of this file in a process of its own (python bench.py --only-extra NAME), so that whatever happens
+    in it cannot take the benchmark's JSON line with it; returns its entry or {"error": ...}."""
+    import subprocess
+    import sys
+    cmd = [sys.executable, os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench.py"), "--only-extra", name]
+    try:
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=timeout)
+        if proc.returncode != 0:
+            return {"error": "exit code %d: %s" % (proc.returncode, proc.stderr.strip()[-300:])}
+        return json.loads(proc.stdout.strip().splitlines()[-1])[name]
+    except Exception as e:
+        return {"error": "%s: %s" % (type(e).__name__, e)}
+
+
 def run(torch, dev):
     out = {}
     for name, fn in (("config1_sc_conv_or1", config1_sc_conv_or1), ("config2_sc_linear", config2_sc_linear),
@@ -379,4 +428,11 @@ def run(torch, dev):
         except Exception as e:
             out[name] = {"error": "%s: %s" % (type(e).__name__, e)}
         torch.cuda.empty_cache()
+    # the reduced-precision step of both networks: float16 convolutions of the vendor library, searched and compiled
+    # per shape on first use -- kept out of this process
+    for name, child in (("config3_tinyconv_train", "config3_tinyconv_autocast_step"),
+                        ("config5_resnet18_train", "config5_resnet18_autocast_step")):
+        res = _in_child_process(child)
+        if isinstance(out.get(name), dict) and "error" not in out[name]:
+            out[name]["sync1_sc_forward_autocast_fp16"] = res.get("sync1_sc_forward_autocast_fp16", res)
     return out

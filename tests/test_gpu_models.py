@@ -154,3 +154,4 @@ def test_config3_tinyconv_training_step_full_batch():
         return (torch.randn(n, 3, 32, 32, generator=g).clamp(-1, 1).cuda(), torch.randint(0, 10, (n,), generator=g).cuda())
 
     _run_config(make_net, make_batch, 256, 8e-3, 4)
+
