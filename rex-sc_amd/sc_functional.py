@@ -213,14 +213,28 @@ def compute_bias_std_coef(or_n, a_bit, a_act, order):
 
 
 # ---- merged surrogate ---------------------------------------------------------------------------
+def _autocast_dtype():
+    """The reduced-precision dtype of an active CUDA autocast region (the reference's half / bfloat16 training,
+    utils_own.py:76-80,127-129), else None."""
+    return torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else None
+
+
 def merged_surrogate_sums(activation, weight, pad_hw, stride):
     """One convolution with the 2*O filters [w_pos ; w_neg], written in the activation's memory order (no
-    conversion pass inside the convolution): -> (w2, s2, outer, inner, channels_last) with s2 laid out
-    [outer][2][inner]."""
+    conversion pass inside the convolution): -> (w2, s2, outer, inner, channels_last, xa) with s2 laid out
+    [outer][2][inner] in float32.  Inside an autocast region the convolution runs in the region's dtype, as the
+    reference's two convolutions do there: w2 and xa (the activation as the convolution took it) are then of that
+    dtype, and s2 holds the reduced-precision sums widened to float32."""
+    lowp = _autocast_dtype()
     with torch.no_grad():
         w2 = _ops.split_weight(weight, channels_last=_ops.is_channels_last(activation))
-        s2, outer, inner, cl = _ops.pair_layout(F.conv2d(activation.detach(), w2, padding=pad_hw, stride=stride))
-    return w2, s2, outer, inner, cl
+        xa = activation.detach()
+        if lowp is not None:
+            w2 = w2.to(lowp)
+            xa = xa.to(lowp)
+        with torch.autocast("cuda", enabled=False):
+            s2, outer, inner, cl = _ops.pair_layout(F.conv2d(xa, w2, padding=pad_hw, stride=stride))
+    return w2, s2, outer, inner, cl, xa
 
 
 class Merged_Surrogate_Conv(torch.autograd.Function):
@@ -237,34 +251,39 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
     Bias_Correct(OR_n(sum_neg)) with those coefficients (:1284-1285), which is what the sync-3 kernel computes.
     Gradients are those of OR_n(conv(x, w_pos)) - OR_n(conv(x, w_neg)) (sync 2, 3: with the bias
     polynomial's derivative), evaluated on the saved sums rounded to binary16 as the reference's
-    backward wrappers do."""
+    backward wrappers do.  Inside an autocast region the forward and backward convolutions run in the region's
+    dtype; the pointwise kernels stay in float32 on the widened sums and the value is float32 (the caller casts)."""
 
     @staticmethod
     def forward(ctx, activation, weight, sc_value, bias_coef, std_coef, or_n, pad_hw, stride, sync, sums):
         if sums is None:
             sums = merged_surrogate_sums(activation, weight, pad_hw, stride)
-        w2, s2, outer, inner, cl = sums
-        ctx.geom = (outer, inner, cl, or_n, tuple(pad_hw), tuple(stride), sync)
+        w2, s2, outer, inner, cl, xa = sums
+        ctx.geom = (outer, inner, cl, or_n, tuple(pad_hw), tuple(stride), sync, activation.dtype)
         if sync >= 2:
-            ctx.save_for_backward(activation, weight, w2, s2, bias_coef)
+            ctx.save_for_backward(xa, weight, w2, s2, bias_coef)
             return _ops.orn_bias_std_pair_forward(s2, outer, inner, cl, bias_coef, std_coef, or_n)
-        ctx.save_for_backward(activation, weight, w2, s2)
+        ctx.save_for_backward(xa, weight, w2, s2)
         return sc_value
 
     @staticmethod
     def backward(ctx, grad_output):
-        outer, inner, cl, or_n, pad_hw, stride, sync = ctx.geom
+        outer, inner, cl, or_n, pad_hw, stride, sync, x_dtype = ctx.geom
         if sync >= 2:
-            activation, weight, w2, s2, bias_coef = ctx.saved_tensors
+            xa, weight, w2, s2, bias_coef = ctx.saved_tensors
             g2 = _ops.orn_bias_std_pair_backward(grad_output, s2, outer, inner, cl, bias_coef, or_n)
         else:
-            activation, weight, w2, s2 = ctx.saved_tensors
+            xa, weight, w2, s2 = ctx.saved_tensors
             g2 = _ops.orn_pair_backward(grad_output, s2, outer, inner, cl, or_n)
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         dx = dw = None
         if need_x or need_w:
-            dx, dw2, _ = torch.ops.aten.convolution_backward(g2, activation, w2, None, stride, pad_hw, (1, 1), False,
+            if g2.dtype != w2.dtype:  # autocast region: the backward convolutions run in its dtype as well
+                g2 = g2.to(w2.dtype)
+            dx, dw2, _ = torch.ops.aten.convolution_backward(g2, xa, w2, None, stride, pad_hw, (1, 1), False,
                                                              (0, 0), 1, (need_x, need_w, False))
+            if need_x and dx.dtype != x_dtype:
+                dx = dx.to(x_dtype)
             if need_w:
                 dw = _ops.merge_weight_grad(dw2, weight).to(weight.dtype)
         return dx, dw, None, None, None, None, None, None, None, None
@@ -307,12 +326,18 @@ def _side_stream(device):
 
 
 def _merged_surrogate_ok(activation, weight, forward, or_n, sync, sc_on, split_output, stride, pad_hw):
-    """Whether conv2d_generic may take the merged path: float32 operands on the GPU, OR-n with a
-    fused kernel, a plain forward value (no split output), and an output shape with a whole number
-    of float4 vectors per polarity block.  REXSC_MERGED_SURROGATE=0 switches it off."""
-    if os.environ.get("REXSC_MERGED_SURROGATE", "1") == "0" or split_output or torch.is_autocast_enabled():
+    """Whether conv2d_generic may take the merged path: float32 operands on the GPU (inside a float16 / bfloat16
+    autocast region the activation may also be of the region's dtype), OR-n with a fused kernel, a plain forward
+    value (no split output), and an output shape with a whole number of float4 vectors per polarity block.
+    REXSC_MERGED_SURROGATE=0 switches it off."""
+    if os.environ.get("REXSC_MERGED_SURROGATE", "1") == "0" or split_output:
         return False
-    if not (activation.is_cuda and weight.is_cuda) or activation.dtype != torch.float32 or weight.dtype != torch.float32:
+    lowp = _autocast_dtype()
+    if lowp is not None and lowp not in (torch.float16, torch.bfloat16):
+        return False
+    if not (activation.is_cuda and weight.is_cuda) or weight.dtype != torch.float32:
+        return False
+    if activation.dtype != torch.float32 and activation.dtype != lowp:
         return False
     if sync == 1:
         if not sc_on or not (forward in ("full_or", "and_2") or (forward[:3] == "or_" and len(forward) == 4)):
@@ -395,15 +420,18 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
     if (sync_override == 3 or has_sc_kernel) and _merged_surrogate_ok(
             activation, weight, forward, or_n, sync_override, sc_on, split_output, stride, pad_hw):
         n = 1 if forward in ("full_or", "and_2") else or_n
+        # the kernels' value is float32; inside an autocast region the reference returns float16 (:1148-1150)
+        as_dtype = lambda t: t if t.dtype == dtype else t.to(dtype)
         if sync_override == 3:
-            return Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride, 3, None)
+            return as_dtype(Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride,
+                                                        3, None))
         if sync_override == 2:
             with torch.no_grad():
                 pos, neg = sc_extension_cuda.conv2d_generic_general_split_acc(
                     activation.data, weight.data, bit_length, LFSR_Length, z_unit, padding, stride,
                     (prec_default, load_unit, load_wait_w), bin_config, gen_config, XNOR, MUX)
                 sums = merged_surrogate_sums(activation, weight, pad_hw, stride)
-                _, s2, outer, inner, cl = sums
+                _, s2, outer, inner, cl, _ = sums
                 # calibration: a_act = OR_n of both sums (one pass over the pair tensor), a_bit = the SC
                 # results in the same element order
                 a_act = _ops.storage_flat(_ops.orn_forward(s2, n), cl)
@@ -412,7 +440,7 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
                 bias_coef[:bias_new.size(0)] = bias_new
                 std_coef[:std_new.size(0)] = std_new
             out = Merged_Surrogate_Conv.apply(activation, weight, None, bias_coef, std_coef, n, pad_hw, stride, 2, sums)
-            return out, bias_coef, std_coef
+            return as_dtype(out), bias_coef, std_coef
 
         def sc_forward():
             # pos / L - neg / L (:1181-1182, 1273-1274, 1317) comes out of the kernel that produces the sums
@@ -422,13 +450,13 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
                                       xnor=_ops.honour_xnor(XNOR), want_value=True)[3]
 
         if not (torch.is_grad_enabled() and (activation.requires_grad or weight.requires_grad)):
-            return sc_forward()  # inference: the surrogate only ever supplies gradients
+            return as_dtype(sc_forward())  # inference: the surrogate only ever supplies gradients
         # The integer kernels (VALU-bound) and the surrogate's float convolution (matrix cores) are
         # independent: the SC forward runs on a second stream of default priority and the two overlap.
         side = _side_stream(activation.device)
         if side is None:
-            return Merged_Surrogate_Conv.apply(activation, weight, sc_forward(), bias_coef, std_coef, n, pad_hw,
-                                               stride, 1, None)
+            return as_dtype(Merged_Surrogate_Conv.apply(activation, weight, sc_forward(), bias_coef, std_coef, n, pad_hw,
+                                                        stride, 1, None))
         cur = torch.cuda.current_stream(activation.device)
         side.wait_stream(cur)
         with torch.cuda.stream(side):
@@ -436,7 +464,7 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
         out = Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride, 1, None)
         cur.wait_stream(side)
         sc_value.record_stream(cur)  # allocated on the side stream, consumed on the caller's
-        return out
+        return as_dtype(out)
 
     result_pos = result_neg = None
     if sc_on:

@@ -219,3 +219,96 @@ def test_sync2_merged_equals_two_convolutions(cl, monkeypatch):
     d = ya - yb
     spread = float(d.std())
     assert 0 < spread < 0.5 and abs(float(d.mean())) < 6 * spread / d.numel() ** 0.5
+
+
+def _run_autocast(monkeypatch, merged, lowp, x, w, pad, stride, forward, sync, channels_last, half_input, bias=None,
+                  std=None):
+    """conv2d_generic inside an autocast region (the reference's reduced-precision step, utils_own.py:127-131)."""
+    import sc_functional as uf
+    monkeypatch.setenv("REXSC_MERGED_SURROGATE", "1" if merged else "0")
+    xt = x.cuda()
+    if half_input:  # what a layer sees behind a reduced-precision convolution and a ReLU
+        xt = xt.to(lowp)
+    if channels_last:
+        xt = xt.contiguous(memory_format=torch.channels_last)
+    xt.requires_grad_(True)
+    wt = w.cuda().requires_grad_(True)
+    torch.manual_seed(11)
+    kw = dict(bit_length=32, generator="lfsr", forward=forward, sync=sync, order=5)
+    if bias is not None:
+        kw.update(bias_coef=bias.cuda(), std_coef=std.cuda())
+    with torch.autocast("cuda", dtype=lowp):
+        out = uf.conv2d_generic(xt, wt, pad, stride, **kw)
+    g = torch.randn(out.shape, generator=torch.Generator().manual_seed(5)).cuda().to(out.dtype)
+    out.backward(g)
+    assert xt.grad.dtype == xt.dtype and wt.grad.dtype == torch.float32
+    return out.detach(), xt.grad.float().cpu(), wt.grad.cpu()
+
+
+def _close_lowp(a, b, what, tol):
+    scale = float(b.abs().max()) + 1e-30
+    err = float((a - b).abs().max())
+    assert err <= tol * scale, "%s: max error %g against scale %g" % (what, err, scale)
+
+
+@pytest.mark.parametrize("case", [CASES[1], CASES[2], CASES[3]])
+@pytest.mark.parametrize("half_input", [False, True])
+def test_merged_path_inside_a_float16_autocast_region(case, half_input, monkeypatch):
+    """Inside an autocast region the merged path runs its convolutions in float16, as the two-convolution path does
+    there; the SC value is the same number and the gradients agree to float16 rounding (both paths round the sums and
+    the convolutions' results to float16; they differ in where the two polarities' data gradients are added)."""
+    N, C, H, W, O, K, pad, stride, cl = case
+    print("merged autocast", case, half_input, flush=True)
+    x, w = _operands(31, N, C, H, W, O, K)
+    import sc_functional as uf
+    calls = []
+    orig = uf.Merged_Surrogate_Conv.apply
+    monkeypatch.setattr(uf.Merged_Surrogate_Conv, "apply", lambda *a: calls.append(1) or orig(*a))
+    ya, gxa, gwa = _run_autocast(monkeypatch, True, torch.float16, x, w, pad, stride, "or_2", 1, cl, half_input)
+    assert calls, "the merged path was not taken inside the autocast region"
+    yb, gxb, gwb = _run_autocast(monkeypatch, False, torch.float16, x, w, pad, stride, "or_2", 1, cl, half_input)
+    assert ya.dtype == torch.float16 and yb.dtype == torch.float16
+    assert torch.equal(ya, yb)  # the SC result: k / 32, exact in float16
+    _close_lowp(gxa, gxb, "grad x", 4e-3)
+    _close_lowp(gwa, gwb, "grad w", 4e-3)
+    # and against the float32 run of the same layer: float16 rounding of sums and gradients only
+    yc, gxc, gwc = _run(monkeypatch, True, x, w, pad, stride, "or_2", 1, cl)
+    assert torch.equal(ya.float().cpu(), yc)
+    _close_lowp(gxa, gxc, "grad x against float32", 1e-2)
+    _close_lowp(gwa, gwc, "grad w against float32", 1e-2)
+
+
+@pytest.mark.parametrize("sync", [3, 2])
+def test_merged_path_autocast_error_injection_and_calibration(sync, monkeypatch):
+    N, C, H, W, O, K, pad, stride, cl = CASES[1]
+    x, w = _operands(32, N, C, H, W, O, K)
+    bias = torch.tensor([0.01, -0.02, 0.005, 0.001, 0, 0])
+    std = torch.zeros(6)  # no noise: the two paths index their noise streams differently per polarity tensor
+    import sc_functional as uf
+    if sync == 3:
+        ya, gxa, gwa = _run_autocast(monkeypatch, True, torch.float16, x, w, pad, stride, "or_2", 3, cl, True, bias, std)
+        yb, gxb, gwb = _run_autocast(monkeypatch, False, torch.float16, x, w, pad, stride, "or_2", 3, cl, True, bias, std)
+        _close_lowp(ya.float().cpu(), yb.float().cpu(), "forward", 4e-3)
+        _close_lowp(gxa, gxb, "grad x", 4e-3)
+        _close_lowp(gwa, gwb, "grad w", 4e-3)
+        return
+    monkeypatch.setenv("REXSC_MERGED_SURROGATE", "1")
+    xt = x.cuda().half().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    wt = w.cuda().requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.float16):
+        out, b, s = uf.conv2d_generic(xt, wt, pad, stride, bit_length=32, generator="lfsr", forward="or_2", sync=2, order=5)
+    out.float().sum().backward()
+    assert out.dtype == torch.float16 and torch.isfinite(out).all()
+    assert torch.isfinite(b).all() and torch.isfinite(s).all() and s.abs().sum() > 0
+    assert torch.isfinite(xt.grad).all() and torch.isfinite(wt.grad).all()
+
+
+def test_merged_path_inside_a_bfloat16_autocast_region(monkeypatch):
+    N, C, H, W, O, K, pad, stride, cl = CASES[1]
+    x, w = _operands(33, N, C, H, W, O, K)
+    ya, gxa, gwa = _run_autocast(monkeypatch, True, torch.bfloat16, x, w, pad, stride, "or_2", 1, cl, True)
+    yc, gxc, gwc = _run(monkeypatch, True, x, w, pad, stride, "or_2", 1, cl)
+    assert ya.dtype == torch.float16  # the reference returns float16 inside any autocast region (utils_functional.py:1148-1150)
+    assert torch.equal(ya.float().cpu(), yc)
+    _close_lowp(gxa, gxc, "grad x against float32", 4e-2)
+    _close_lowp(gwa, gwc, "grad w against float32", 4e-2)
