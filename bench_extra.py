@@ -25,7 +25,7 @@ VALU_PEAK_4CYCLE = 256 * 4 * 16 * 2.4e9
 HBM_PEAK = 8.0e12
 ROTATE_BYTES = 1.25 * 2 ** 30  # distinct bytes touched before a buffer is used again
 
-SC_KERNELS = ("sc_compute", "sc_finalize", "sng_")
+SC_KERNELS = ("sc_compute", "sc_finalize", "sng_", "fold_")
 STREAM_KERNELS = ("orn_", "sc_counts_to_float", "quantize", "split_weight", "merge_weight_grad", "calib_stats",
                   "fixed_")
 

@@ -983,21 +983,45 @@ int weights_snapshot(const float *w, float *snapshot, size_t n, unsigned long lo
 }
 
 // ---- tap folding --------------------------------------------------------------------------------
-// One thread per (output pixel, slot): lanes are neighbouring output pixels, so every tap's load is coalesced.
+// One thread per output pixel and group of FOLD_SLOTS slots: lanes are neighbouring output pixels, so every tap's
+// load is coalesced.  KH, KW > 0: kernel size known at compile time, so that all loads of a thread are in flight
+// together (with run-time bounds every tap waits for the one before it: a chain of KH*KW cache latencies); 0: any size.
+constexpr int FOLD_SLOTS = 4;
+template <int KH_T, int KW_T>
 __global__ __launch_bounds__(256) void fold_act_kernel(const uint32_t *__restrict__ A, uint32_t *__restrict__ A2, long a_stride,
-                                                       long a2_stride, unsigned M, int Hp, int Wp, int Ho, int Wo, int KH, int KW,
-                                                       int s0, int s1, int C)
+                                                       long a2_stride, unsigned M, int n_slots, int Hp, int Wp, int Ho, int Wo,
+                                                       int KH_R, int KW_R, int s0, int s1, int C)
 {
     const unsigned m = blockIdx.x * 256 + threadIdx.x;
     if (m >= M) return;
+    const int KH = KH_T ? KH_T : KH_R, KW = KW_T ? KW_T : KW_R;
     const unsigned HoWo = (unsigned)Ho * Wo;
     const unsigned n = m / HoWo, r = m - n * HoWo;
     const unsigned yo = r / (unsigned)Wo, xo = r - yo * (unsigned)Wo;
-    const uint32_t *src = A + (long)blockIdx.y * a_stride + ((long)n * Hp + yo * s0) * Wp + xo * s1;
-    uint32_t word = 0;
-    for (int ky = 0; ky < KH; ky++)
-        for (int kx = 0; kx < KW; kx++) word |= src[ky * Wp + kx] << ((ky * KW + kx) * C);
-    A2[(long)blockIdx.y * a2_stride + m] = word;
+    const int slot0 = blockIdx.y * FOLD_SLOTS;
+    const uint32_t *src = A + (long)slot0 * a_stride + ((long)n * Hp + yo * s0) * Wp + xo * s1;
+    uint32_t *dst = A2 + (long)slot0 * a2_stride + m;
+    if (KH_T && slot0 + FOLD_SLOTS <= n_slots) {
+        uint32_t v[FOLD_SLOTS][KH_T ? KH_T * KW_T : 1];
+#pragma unroll
+        for (int q = 0; q < FOLD_SLOTS; q++)
+#pragma unroll
+            for (int t = 0; t < KH_T * KW_T; t++) v[q][t] = src[q * a_stride + (t / KW_T) * Wp + (t % KW_T)];
+#pragma unroll
+        for (int q = 0; q < FOLD_SLOTS; q++) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int t = 0; t < KH_T * KW_T; t++) word |= v[q][t] << (t * C);
+            dst[q * a2_stride] = word;
+        }
+        return;
+    }
+    for (int q = 0; q < FOLD_SLOTS && slot0 + q < n_slots; q++) {
+        uint32_t word = 0;
+        for (int ky = 0; ky < KH; ky++)
+            for (int kx = 0; kx < KW; kx++) word |= src[q * a_stride + ky * Wp + kx] << ((ky * KW + kx) * C);
+        dst[q * a2_stride] = word;
+    }
 }
 
 __global__ __launch_bounds__(256) void fold_weight_kernel(const uint32_t *__restrict__ Wst, uint32_t *__restrict__ W2, int n_slots,
@@ -1025,8 +1049,15 @@ int fold_activation_streams(const uint32_t *A, uint32_t *A2, int n_slots, long a
     const long M = (long)N * Ho * Wo;
     REXSC_CHECK_ARG(C * KH * KW <= 32 && M > 0 && M < (1L << 31) && n_slots <= 65535, "tap folding: shape out of range");
     ProfScope prof("fold_act", 4.0 * n_slots * ((double)N * Hp * Wp + (double)M), stream);
-    hipLaunchKernelGGL(fold_act_kernel, dim3((unsigned)((M + 255) / 256), (unsigned)n_slots), dim3(256), 0, stream, A, A2, a_stride,
-                       a2_stride, (unsigned)M, Hp, Wp, Ho, Wo, KH, KW, s0, s1, C);
+    const dim3 grid((unsigned)((M + 255) / 256), (unsigned)ceil_div(n_slots, FOLD_SLOTS));
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(256), 0, stream, A, A2, a_stride, a2_stride, (unsigned)M, n_slots, Hp, Wp, Ho, Wo,
+                           KH, KW, s0, s1, C);
+    };
+    if (KH == 3 && KW == 3) launch(fold_act_kernel<3, 3>);
+    else if (KH == 5 && KW == 5) launch(fold_act_kernel<5, 5>);
+    else if (KH == 2 && KW == 2) launch(fold_act_kernel<2, 2>);
+    else launch(fold_act_kernel<0, 0>);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }
