@@ -153,15 +153,17 @@ def config2_sc_linear(torch, dev):
     return out
 
 
-def _train_flavours(torch, dev, net, make_batch, batch, steps, lr, only_autocast=False):
-    """Training steps as utils_own.py:96-171 runs them: sync 1 / 3 / 2 in float32; with only_autocast, sync 1 under
+def _train_flavours(torch, dev, net, make_batch, batch, steps, lr, only=None):
+    """Training steps as utils_own.py:96-171 runs them: sync 1 / 3 / 2 in float32; only="autocast": sync 1 under
     float16 autocast with a gradient scaler instead (the reference's `torch_type != torch.float32` branch,
-    :127-131,156-165)."""
+    :127-131,156-165); only="sync1": the float32 sync-1 flavour alone (for profiler runs)."""
     import torch.nn.functional as F
     opt = torch.optim.Adam(net.parameters(), lr=lr, weight_decay=1e-4)
+    only_autocast = only == "autocast"
     scaler = torch.amp.GradScaler("cuda") if only_autocast else None
     out = {}
     flavours = ((("sync1_sc_forward_autocast_fp16", 1, 1.0),) if only_autocast else
+                (("sync1_sc_forward", 1, 1.0),) if only == "sync1" else
                 (("sync1_sc_forward", 1, 1.0), ("sync3_error_injection", 3, 1.0), ("sync2_calibration_half_batch", 2, 0.5)))
     for name, sync, frac in flavours:
         n = max(1, int(batch * frac))
@@ -193,7 +195,7 @@ def _train_flavours(torch, dev, net, make_batch, batch, steps, lr, only_autocast
     return out
 
 
-def config3_tinyconv_step(torch, dev, only_autocast=False):
+def config3_tinyconv_step(torch, dev, only=None):
     from sc_models import TinyConvSC
     torch.manual_seed(3)
     net = TinyConvSC(forward="or_3", err=6).to(dev)
@@ -203,14 +205,14 @@ def config3_tinyconv_step(torch, dev, only_autocast=False):
         return (torch.randn(n, 3, 32, 32, generator=g).clamp(-1, 1).to(dev),
                 torch.randint(0, 10, (n,), generator=g).to(dev))
 
-    res = _train_flavours(torch, dev, net, make_batch, 256, 10, 8e-3, only_autocast)
+    res = _train_flavours(torch, dev, net, make_batch, 256, 10, 8e-3, only)
     res["workload"] = ("TinyConv-style training step, batch 256, 3x32x32, conv3x3 3-32-32-pool-64-64-pool-fc10, "
                        "OR-3, 64-bit streams, Adam")
     return res
 
 
 def config3_tinyconv_autocast_step(torch, dev):
-    return config3_tinyconv_step(torch, dev, only_autocast=True)
+    return config3_tinyconv_step(torch, dev, only="autocast")
 
 
 def _rotating_sets(nbytes_per_set):
@@ -280,10 +282,18 @@ def config4_fixed_conv(torch, dev):
 
 
 def config5_resnet18_autocast_step(torch, dev):
-    return config5_resnet18_step(torch, dev, only_autocast=True)
+    return config5_resnet18_step(torch, dev, only="autocast")
 
 
-def config5_resnet18_step(torch, dev, batch=64, only_autocast=False):
+def config5_resnet18_sync1_step(torch, dev):
+    return config5_resnet18_step(torch, dev, only="sync1")
+
+
+def config3_tinyconv_sync1_step(torch, dev):
+    return config3_tinyconv_step(torch, dev, only="sync1")
+
+
+def config5_resnet18_step(torch, dev, batch=64, only=None):
     from sc_models import ResNet18SC
     torch.manual_seed(5)
     net = ResNet18SC(forward="or_2", err=5).to(dev).to(memory_format=torch.channels_last)
@@ -293,10 +303,10 @@ def config5_resnet18_step(torch, dev, batch=64, only_autocast=False):
         return (torch.randn(n, 3, 224, 224, generator=g).to(dev).contiguous(memory_format=torch.channels_last),
                 torch.randint(0, 1000, (n,), generator=g).to(dev))
 
-    res = _train_flavours(torch, dev, net, make_batch, batch, 5, 1e-3, only_autocast)
+    res = _train_flavours(torch, dev, net, make_batch, batch, 5, 1e-3, only)
     res["workload"] = ("ResNet-18 SC training step, batch %d, 3x224x224, channels_last, OR-2, 32-bit streams, "
                        "float stem/fc, Adam" % batch)
-    if only_autocast:
+    if only:
         return res
     # evaluation: weights frozen, the layers reuse their weight streams from call to call
     net.eval()
