@@ -230,6 +230,12 @@ int rexsc_orn_bias_std_backward(const float *grad_out, const float *x, const flo
  * the same noise stream per element of y.  g2 has s2's layout (gradient of the merged convolution). */
 int rexsc_orn_pair_backward(const float *grad_out, const float *s2, float *g2, size_t outer, size_t inner,
                             int or_n, int half_input, rexsc_stream_t stream);
+/* The same with grad_out, s2 and g2 stored as binary16 (8-byte aligned), for callers inside a float16 autocast
+ * region, where the convolutions on either side of this kernel produce and consume float16 (utils_own.py:127-131;
+ * the wrappers of sc_cuda_pw.cu:767-832 take such tensors and widen them).  Arithmetic in float32, one rounding on
+ * the store: equal to widening, rexsc_orn_pair_backward with half_input = 1, and a cast of g2 to float16. */
+int rexsc_orn_pair_backward_f16(const uint16_t *grad_out, const uint16_t *s2, uint16_t *g2, size_t outer, size_t inner,
+                                int or_n, rexsc_stream_t stream);
 int rexsc_orn_bias_std_pair_forward(const float *s2, const float *bias_coef, const float *std_coef, float *y,
                                     size_t outer, size_t inner, int or_n, uint64_t seed, uint64_t offset,
                                     const uint64_t *offset_dev, rexsc_stream_t stream);

@@ -79,6 +79,7 @@ SIGNATURES = {
     "rexsc_orn_bias_std_forward_f16": (_int, [_vp, _vp, _vp, _vp, _sz, _int, _u64, _u64, _vp, _vp]),
     "rexsc_orn_bias_std_backward": (_int, [_vp, _vp, _vp, _vp, _sz, _int, _int, _vp]),
     "rexsc_orn_pair_backward": (_int, [_vp, _vp, _vp, _sz, _sz, _int, _int, _vp]),
+    "rexsc_orn_pair_backward_f16": (_int, [_vp, _vp, _vp, _sz, _sz, _int, _vp]),
     "rexsc_orn_bias_std_pair_forward": (_int, [_vp, _vp, _vp, _vp, _sz, _sz, _int, _u64, _u64, _vp, _vp]),
     "rexsc_orn_bias_std_pair_backward": (_int, [_vp, _vp, _vp, _vp, _sz, _sz, _int, _int, _vp]),
     "rexsc_sc_counts_to_float": (_int, [_vp, _vp, _vp, _sz, _int, _vp]),

@@ -62,9 +62,11 @@ def is_channels_last(t):
     return s[1] == 1 and s[1] * s[2] * s[3] != 1
 
 
-def _as_layout(t, channels_last):
+def _as_layout(t, channels_last, keep_half=False):
+    """Dense float32 copy (or t itself) in the requested memory order, 16-byte aligned; keep_half: a float16 tensor
+    stays float16."""
     t = t.detach()
-    if t.dtype != torch.float32:
+    if t.dtype != torch.float32 and not (keep_half and t.dtype == torch.float16):
         t = t.float()
     fmt = torch.channels_last if channels_last else torch.contiguous_format
     t = t.contiguous(memory_format=fmt)
@@ -342,10 +344,11 @@ def _dense_f32(t):
 
 
 def _like_layout(t, ref):
-    """float32 copy of t laid out with ref's strides (the kernels index raw storage)."""
+    """Copy of t in ref's dtype (float32, or float16 for the binary16 kernels) laid out with ref's strides (the
+    kernels index raw storage)."""
     t = t.detach()
-    if t.dtype != torch.float32:
-        t = t.float()
+    if t.dtype != ref.dtype:
+        t = t.to(ref.dtype)
     if t.stride() != ref.stride() or t.data_ptr() % 16:
         out = torch.empty_like(ref)
         out.copy_(t)
@@ -481,10 +484,11 @@ def orn_bias_std_backward(grad_output, x, bias_coef, or_n, half_input=True):
 
 # ---- merged surrogate (polarity-pair layout) ---------------------------------------------------
 
-def pair_layout(s2):
+def pair_layout(s2, keep_half=False):
     """s2 = conv / linear output with 2*O channels (O positive, then O negative).  Returns
     (s2 dense, outer, inner, channels_last) for the [outer][2][inner] view of its storage, re-laying
-    the tensor out if its own layout has no inner % 4 == 0 view; None if neither layout has one."""
+    the tensor out if its own layout has no inner % 4 == 0 view; None if neither layout has one.
+    The result is float32 unless keep_half and s2 is float16 (for orn_pair_backward's binary16 kernel)."""
     s2 = s2.detach()
     O = s2.size(1) // 2
     if s2.dim() == 2:
@@ -493,26 +497,32 @@ def pair_layout(s2):
     ok_cl, ok_nchw = O % 4 == 0, (O * H * W) % 4 == 0
     is_cl = s2.is_contiguous(memory_format=torch.channels_last) and not s2.is_contiguous()
     if (is_cl and ok_cl) or (not ok_nchw and ok_cl):
-        return _as_layout(s2, True), N * H * W, O, True
+        return _as_layout(s2, True, keep_half), N * H * W, O, True
     if ok_nchw:
-        return _as_layout(s2, False), N, O * H * W, False
+        return _as_layout(s2, False, keep_half), N, O * H * W, False
     return None
 
 
-def _pair_result_like(s2, channels_last):
+def _pair_result_like(s2, channels_last, dtype=torch.float32):
     if s2.dim() == 2:
-        return torch.empty((s2.size(0), s2.size(1) // 2), dtype=torch.float32, device=s2.device)
+        return torch.empty((s2.size(0), s2.size(1) // 2), dtype=dtype, device=s2.device)
     N, O2, H, W = s2.shape
-    return _empty_out((N, O2 // 2, H, W), torch.float32, s2.device, channels_last)
+    return _empty_out((N, O2 // 2, H, W), dtype, s2.device, channels_last)
 
 
 def orn_pair_backward(grad_output, s2, outer, inner, channels_last, or_n, half_input=True):
-    y_like = _pair_result_like(s2, channels_last)
+    """Gradient of the merged convolution's output.  s2 float32: float32 in and out; s2 float16 (pair_layout with
+    keep_half, inside a float16 autocast region): the binary16 kernel, float16 in and out."""
+    half = s2.dtype == torch.float16
+    y_like = _pair_result_like(s2, channels_last, s2.dtype)
     g = _like_layout(grad_output, y_like)
     g2 = torch.empty_like(s2)
     with torch.cuda.device(s2.device):
-        rc = _lib.lib().rexsc_orn_pair_backward(_ptr(g), _ptr(s2), _ptr(g2), outer, inner, int(or_n), int(half_input),
-                                                _stream())
+        if half:
+            rc = _lib.lib().rexsc_orn_pair_backward_f16(_ptr(g), _ptr(s2), _ptr(g2), outer, inner, int(or_n), _stream())
+        else:
+            rc = _lib.lib().rexsc_orn_pair_backward(_ptr(g), _ptr(s2), _ptr(g2), outer, inner, int(or_n), int(half_input),
+                                                    _stream())
         _lib.check(rc, "rexsc_orn_pair_backward")
     return g2
 

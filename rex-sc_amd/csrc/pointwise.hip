@@ -352,19 +352,43 @@ __device__ __forceinline__ size_t pair_vec_offset(size_t q, unsigned inner4)
     return (size_t)q + (size_t)o * inner4;   // = o * 2 * inner4 + (q - o * inner4)
 }
 
-template <int N>
-__global__ __launch_bounds__(PW_THREADS) void orn_pair_backward_kernel(const float *__restrict__ g,
-                                                                       const float *__restrict__ s2,
-                                                                       float *__restrict__ g2, size_t nvec,
+// Four neighbouring elements of a float32 or binary16 tensor (16- or 8-byte access), widened to float32.
+template <typename T> struct Vec4Io;
+template <> struct Vec4Io<float> {
+    static __device__ __forceinline__ float4 load(const float *p, size_t v) { return reinterpret_cast<const float4 *>(p)[v]; }
+    static __device__ __forceinline__ void store(float *p, size_t v, float4 x) { reinterpret_cast<float4 *>(p)[v] = x; }
+};
+template <> struct Vec4Io<__half> {
+    static __device__ __forceinline__ float4 load(const __half *p, size_t v)
+    {
+        const uint2 raw = reinterpret_cast<const uint2 *>(p)[v];
+        const __half2 lo = *reinterpret_cast<const __half2 *>(&raw.x), hi = *reinterpret_cast<const __half2 *>(&raw.y);
+        return make_float4(__low2float(lo), __high2float(lo), __low2float(hi), __high2float(hi));
+    }
+    static __device__ __forceinline__ void store(__half *p, size_t v, float4 x)
+    {   // round to nearest even, as a tensor cast to float16 does
+        const __half2 lo = __floats2half2_rn(x.x, x.y), hi = __floats2half2_rn(x.z, x.w);
+        uint2 raw;
+        raw.x = *reinterpret_cast<const uint32_t *>(&lo);
+        raw.y = *reinterpret_cast<const uint32_t *>(&hi);
+        reinterpret_cast<uint2 *>(p)[v] = raw;
+    }
+};
+
+// T = float: the tensors as the float32 surrogate leaves them.  T = __half: all three tensors in binary16, as inside
+// a float16 autocast region (the arithmetic stays float32; results are rounded once, on the store).
+template <int N, typename T>
+__global__ __launch_bounds__(PW_THREADS) void orn_pair_backward_kernel(const T *__restrict__ g, const T *__restrict__ s2,
+                                                                       T *__restrict__ g2, size_t nvec,
                                                                        unsigned inner4, int half_input)
 {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
         const size_t off = pair_vec_offset(q, inner4);
-        float4 a = reinterpret_cast<const float4 *>(s2)[off];
-        float4 c = reinterpret_cast<const float4 *>(s2)[off + inner4];
-        const float4 gg = reinterpret_cast<const float4 *>(g)[q];
-        if (half_input) {
+        float4 a = Vec4Io<T>::load(s2, off);
+        float4 c = Vec4Io<T>::load(s2, off + inner4);
+        const float4 gg = Vec4Io<T>::load(g, q);
+        if (half_input && sizeof(T) == 4) {
             a.x = round_half(a.x); a.y = round_half(a.y); a.z = round_half(a.z); a.w = round_half(a.w);
             c.x = round_half(c.x); c.y = round_half(c.y); c.z = round_half(c.z); c.w = round_half(c.w);
         }
@@ -373,8 +397,8 @@ __global__ __launch_bounds__(PW_THREADS) void orn_pair_backward_kernel(const flo
         rp.y = orn_bwd<N>(gg.y, a.y); rn.y = orn_bwd<N>(-gg.y, c.y);
         rp.z = orn_bwd<N>(gg.z, a.z); rn.z = orn_bwd<N>(-gg.z, c.z);
         rp.w = orn_bwd<N>(gg.w, a.w); rn.w = orn_bwd<N>(-gg.w, c.w);
-        reinterpret_cast<float4 *>(g2)[off] = rp;
-        reinterpret_cast<float4 *>(g2)[off + inner4] = rn;
+        Vec4Io<T>::store(g2, off, rp);
+        Vec4Io<T>::store(g2, off + inner4, rn);
     }
 }
 
@@ -747,8 +771,29 @@ extern "C" int rexsc_orn_pair_backward(const float *g, const float *s2, float *g
     REXSC_CHECK_ARG(g && s2 && g2, "null pointer");
     const int grid = pw_grid(nvec);
     ProfScope prof("orn_pair_backward", 20.0 * outer * inner, stream);
-    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL(orn_pair_backward_kernel<N>, dim3(grid), dim3(PW_THREADS), 0, stream, g,
-                                               s2, g2, nvec, (unsigned)(inner / 4), half_input));
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL((orn_pair_backward_kernel<N, float>), dim3(grid), dim3(PW_THREADS), 0, stream,
+                                               g, s2, g2, nvec, (unsigned)(inner / 4), half_input));
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+// The same on binary16 tensors (grad_out, s2 and g2 all float16; 8-byte aligned): what the merged surrogate holds
+// inside a float16 autocast region.  Equal to widening the inputs, calling rexsc_orn_pair_backward and rounding g2.
+extern "C" int rexsc_orn_pair_backward_f16(const uint16_t *g, const uint16_t *s2, uint16_t *g2, size_t outer, size_t inner,
+                                           int or_n, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(or_n >= 1 && or_n <= 4, "or_n must be 1..4 (got %d)", or_n);
+    if (int rc = check_pair(outer, inner)) return rc;
+    const size_t nvec = outer * inner / 4;
+    if (nvec == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(g && s2 && g2, "null pointer");
+    REXSC_CHECK_ARG(((uintptr_t)g | (uintptr_t)s2 | (uintptr_t)g2) % 8 == 0, "float16 tensors must be 8-byte aligned");
+    const int grid = pw_grid(nvec);
+    ProfScope prof("orn_pair_backward", 10.0 * outer * inner, stream);
+    REXSC_OR_N_SWITCH(or_n, hipLaunchKernelGGL((orn_pair_backward_kernel<N, __half>), dim3(grid), dim3(PW_THREADS), 0, stream,
+                                               (const __half *)g, (const __half *)s2, (__half *)g2, nvec,
+                                               (unsigned)(inner / 4), 1));
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

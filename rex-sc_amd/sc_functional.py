@@ -219,12 +219,13 @@ def _autocast_dtype():
     return torch.get_autocast_dtype("cuda") if torch.is_autocast_enabled() else None
 
 
-def merged_surrogate_sums(activation, weight, pad_hw, stride):
+def merged_surrogate_sums(activation, weight, pad_hw, stride, keep_half=False):
     """One convolution with the 2*O filters [w_pos ; w_neg], written in the activation's memory order (no
     conversion pass inside the convolution): -> (w2, s2, outer, inner, channels_last, xa) with s2 laid out
     [outer][2][inner] in float32.  Inside an autocast region the convolution runs in the region's dtype, as the
     reference's two convolutions do there: w2 and xa (the activation as the convolution took it) are then of that
-    dtype, and s2 holds the reduced-precision sums widened to float32."""
+    dtype, and s2 holds the reduced-precision sums widened to float32 -- or, with keep_half in a float16 region, as
+    they are (for the backward kernel that reads and writes float16)."""
     lowp = _autocast_dtype()
     with torch.no_grad():
         w2 = _ops.split_weight(weight, channels_last=_ops.is_channels_last(activation))
@@ -233,7 +234,8 @@ def merged_surrogate_sums(activation, weight, pad_hw, stride):
             w2 = w2.to(lowp)
             xa = xa.to(lowp)
         with torch.autocast("cuda", enabled=False):
-            s2, outer, inner, cl = _ops.pair_layout(F.conv2d(xa, w2, padding=pad_hw, stride=stride))
+            s2, outer, inner, cl = _ops.pair_layout(F.conv2d(xa, w2, padding=pad_hw, stride=stride),
+                                                    keep_half=keep_half and lowp == torch.float16)
     return w2, s2, outer, inner, cl, xa
 
 
@@ -257,7 +259,8 @@ class Merged_Surrogate_Conv(torch.autograd.Function):
     @staticmethod
     def forward(ctx, activation, weight, sc_value, bias_coef, std_coef, or_n, pad_hw, stride, sync, sums):
         if sums is None:
-            sums = merged_surrogate_sums(activation, weight, pad_hw, stride)
+            # sync 1 never evaluates the forward kernels on the sums: they can stay in the convolution's float16
+            sums = merged_surrogate_sums(activation, weight, pad_hw, stride, keep_half=(sync == 1))
         w2, s2, outer, inner, cl, xa = sums
         ctx.geom = (outer, inner, cl, or_n, tuple(pad_hw), tuple(stride), sync, activation.dtype)
         if sync >= 2:
@@ -454,17 +457,19 @@ def conv2d_generic(activation, weight, padding, stride, **kwargs):
         # The integer kernels (VALU-bound) and the surrogate's float convolution (matrix cores) are
         # independent: the SC forward runs on a second stream of default priority and the two overlap.
         side = _side_stream(activation.device)
+        # (the value is cast where it is produced, so that the Function's output -- and with it the gradient that
+        # comes back -- has the region's dtype without a cast node of autograd's in between)
         if side is None:
-            return as_dtype(Merged_Surrogate_Conv.apply(activation, weight, sc_forward(), bias_coef, std_coef, n, pad_hw,
-                                                        stride, 1, None))
+            return Merged_Surrogate_Conv.apply(activation, weight, as_dtype(sc_forward()), bias_coef, std_coef, n, pad_hw,
+                                               stride, 1, None)
         cur = torch.cuda.current_stream(activation.device)
         side.wait_stream(cur)
         with torch.cuda.stream(side):
-            sc_value = sc_forward()
+            sc_value = as_dtype(sc_forward())
         out = Merged_Surrogate_Conv.apply(activation, weight, sc_value, bias_coef, std_coef, n, pad_hw, stride, 1, None)
         cur.wait_stream(side)
         sc_value.record_stream(cur)  # allocated on the side stream, consumed on the caller's
-        return as_dtype(out)
+        return out
 
     result_pos = result_neg = None
     if sc_on:

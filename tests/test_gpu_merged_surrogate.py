@@ -312,3 +312,25 @@ def test_merged_path_inside_a_bfloat16_autocast_region(monkeypatch):
     assert torch.equal(ya.float().cpu(), yc)
     _close_lowp(gxa, gxc, "grad x against float32", 4e-2)
     _close_lowp(gwa, gwc, "grad w against float32", 4e-2)
+
+
+@pytest.mark.parametrize("or_n", [1, 2, 3, 4])
+@pytest.mark.parametrize("cl", [False, True])
+def test_pair_backward_on_float16_tensors_equals_widen_compute_round(or_n, cl):
+    """rexsc_orn_pair_backward_f16 (all three tensors binary16) = widen, rexsc_orn_pair_backward, round: bit for bit."""
+    import _ops
+    g = torch.Generator().manual_seed(40 + or_n)
+    N, O, H, W = 3, 8, 5, 6
+    s2 = (torch.rand(N, 2 * O, H, W, generator=g) * 6).half().cuda()
+    go = (torch.randn(N, O, H, W, generator=g) * 3).half().cuda()
+    if cl:
+        s2 = s2.contiguous(memory_format=torch.channels_last)
+        go = go.contiguous(memory_format=torch.channels_last)
+    s2h, outer, inner, c = _ops.pair_layout(s2, keep_half=True)
+    assert s2h.dtype == torch.float16
+    got = _ops.orn_pair_backward(go, s2h, outer, inner, c, or_n)
+    s2f, outer2, inner2, c2 = _ops.pair_layout(s2)
+    assert s2f.dtype == torch.float32 and (outer2, inner2, c2) == (outer, inner, c)
+    want = _ops.orn_pair_backward(go, s2f, outer2, inner2, c2, or_n)
+    assert got.dtype == torch.float16 and want.dtype == torch.float32
+    assert torch.equal(got, want.half()) and float(want.abs().max()) > 0
