@@ -263,6 +263,9 @@ int rexsc_merge_weight_grad(const float *dw2, const float *w, float *dw, size_t 
  * 0 <= prec <= 16: the mul / round / clamp / div passes of `quantize` (utils_functional.py:93-104, the
  * forward of QuantizeGrad :117-123) in one.  n float32 elements of any dense layout; y may alias x. */
 int rexsc_quantize(const float *x, float *y, size_t n, int prec, rexsc_stream_t stream);
+/* The same on binary16 tensors (8-byte aligned), prec 0..10: what QuantizeGrad sees inside a float16 autocast region
+ * (utils_own.py:127-131); equal to the reference's four float16 tensor passes there. */
+int rexsc_quantize_f16(const uint16_t *x, uint16_t *y, size_t n, int prec, rexsc_stream_t stream);
 
 /* Philox4x32-10 block function on the host (for known-answer tests of the generator). */
 void rexsc_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);

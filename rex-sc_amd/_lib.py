@@ -86,6 +86,7 @@ SIGNATURES = {
     "rexsc_split_weight": (_int, [_vp, _vp, _sz, _sz, _sz, _int, _int, _vp]),
     "rexsc_merge_weight_grad": (_int, [_vp, _vp, _vp, _sz, _sz, _sz, _int, _int, _vp]),
     "rexsc_quantize": (_int, [_vp, _vp, _sz, _int, _vp]),
+    "rexsc_quantize_f16": (_int, [_vp, _vp, _sz, _int, _vp]),
     "rexsc_philox4x32_10": (None, [ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
                                    ctypes.POINTER(ctypes.c_uint32)]),
     "rexsc_fixed_conv2d_workspace_bytes": (_sz, [ctypes.POINTER(FixedDesc)]),

@@ -634,8 +634,20 @@ def merge_weight_grad(dw2, w):
 
 
 def quantize(x, prec):
-    """clamp(round(x * 2^prec), +-(2^prec - 1)) / 2^prec in one pass, in x's layout."""
+    """clamp(round(x * 2^prec), +-(2^prec - 1)) / 2^prec in one pass, in x's layout (float16 stays float16 for
+    prec <= 10; everything else is computed and returned in float32)."""
     _require_cuda(x)
+    if x.dtype == torch.float16 and 0 <= int(prec) <= 10:
+        xd = x.detach()
+        if not (xd.is_contiguous() or (xd.dim() == 4 and xd.is_contiguous(memory_format=torch.channels_last))):
+            xd = xd.contiguous()
+        if xd.data_ptr() % 8:
+            xd = xd.clone(memory_format=torch.preserve_format)
+        y = torch.empty_like(xd)
+        with torch.cuda.device(xd.device):
+            rc = _lib.lib().rexsc_quantize_f16(_ptr(xd), _ptr(y), xd.numel(), int(prec), _stream())
+            _lib.check(rc, "rexsc_quantize_f16")
+        return y
     xd = _dense_f32(x)
     y = torch.empty_like(xd)
     with torch.cuda.device(xd.device):

@@ -539,6 +539,25 @@ __global__ __launch_bounds__(PW_THREADS) void quantize_kernel(const float *__res
     if (i < n) y[i] = quantize_one(x[i], scale, inv_scale, lim);
 }
 
+// The same on binary16 tensors: widened, quantised in float32, rounded back (exact: the results are multiples of
+// 2^-prec below one).  Equal to the four float16 tensor passes for prec <= 10, where every intermediate is
+// representable in binary16 or saturates the same way.
+__global__ __launch_bounds__(PW_THREADS) void quantize_f16_kernel(const __half *__restrict__ x, __half *__restrict__ y, size_t n,
+                                                                 float scale, float inv_scale, float lim)
+{
+    const size_t nvec = n / 4;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < nvec; q += stride) {
+        const float4 v = Vec4Io<__half>::load(x, q);
+        float4 r;
+        r.x = quantize_one(v.x, scale, inv_scale, lim); r.y = quantize_one(v.y, scale, inv_scale, lim);
+        r.z = quantize_one(v.z, scale, inv_scale, lim); r.w = quantize_one(v.w, scale, inv_scale, lim);
+        Vec4Io<__half>::store(y, q, r);
+    }
+    const size_t i = nvec * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = __float2half(quantize_one(__half2float(x[i]), scale, inv_scale, lim));
+}
+
 // Calibration statistics: per window k, count / sum / sum of squares of (a_bit - a_act) over
 // the elements with lo[k] <= a_act < hi[k].  Windows may overlap.
 constexpr int CAL_MAX_WIN = 64;
@@ -878,6 +897,22 @@ extern "C" int rexsc_merge_weight_grad(const float *dw2, const float *w, float *
     hipLaunchKernelGGL(merge_weight_grad_kernel, dim3((unsigned)((n + PW_THREADS - 1) / PW_THREADS)), dim3(PW_THREADS),
                        0, stream, dw2, w, dw, n, (unsigned)in_channels, (unsigned)taps, dw2_channels_last,
                        w_channels_last);
+    REXSC_CHECK_HIP(hipGetLastError());
+    return REXSC_OK;
+}
+
+extern "C" int rexsc_quantize_f16(const uint16_t *x, uint16_t *y, size_t n, int prec, rexsc_stream_t stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    REXSC_CHECK_ARG(prec >= 0 && prec <= 10, "prec must be 0..10 for float16 tensors (got %d)", prec);
+    if (n == 0) return REXSC_OK;
+    REXSC_CHECK_ARG(x && y, "null pointer");
+    REXSC_CHECK_ARG(((uintptr_t)x | (uintptr_t)y) % 8 == 0, "float16 tensors must be 8-byte aligned");
+    const float scale = (float)(1u << prec);
+    const int grid = pw_grid((n + 3) / 4);
+    ProfScope prof("quantize", 4.0 * n, stream);
+    hipLaunchKernelGGL(quantize_f16_kernel, dim3(grid), dim3(PW_THREADS), 0, stream, (const __half *)x, (__half *)y, n, scale,
+                       1.0f / scale, scale - 1.0f);
     REXSC_CHECK_HIP(hipGetLastError());
     return REXSC_OK;
 }

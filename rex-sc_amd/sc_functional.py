@@ -51,7 +51,8 @@ def update_sync(model, sync=1):
 def quantize(input, prec=8):
     """(x * 2^prec).round().clamp(+-(2^prec - 1)) / 2^prec  (utils_functional.py:93-104, prune = 0)."""
     if prec <= 16:
-        if (input.is_cuda and input.dtype == torch.float32 and prec >= 0 and not torch.is_grad_enabled()
+        if (input.is_cuda and prec >= 0 and not torch.is_grad_enabled()
+                and (input.dtype == torch.float32 or (input.dtype == torch.float16 and prec <= 10))
                 and (input.is_contiguous() or (input.dim() == 4
                                                and input.is_contiguous(memory_format=torch.channels_last)))):
             return _ops.quantize(input, prec)  # the same four passes as one kernel

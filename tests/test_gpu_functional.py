@@ -227,3 +227,27 @@ def test_fused_quantize_equals_the_four_torch_passes(prec):
     assert torch.equal(y4, (x4.detach() * s).round().clamp(-s + 1, s - 1) / s)
     y4.backward(torch.ones_like(y4))
     assert torch.equal(x4.grad, torch.ones_like(x4))
+
+
+@pytest.mark.parametrize("prec", [0, 1, 5, 7, 10])
+def test_fused_quantize_on_float16_equals_the_four_float16_passes(prec):
+    """Inside a float16 autocast region QuantizeGrad sees float16 activations: every float16 bit pattern through
+    rexsc_quantize_f16 against mul / round / clamp / div on the float16 tensor, bit for bit."""
+    import _ops
+    import sc_functional as uf
+    s = 2.0 ** prec
+    x = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16).view(torch.float16).cuda()  # all 65536 patterns
+    want = (x * s).round().clamp(-s + 1, s - 1) / s
+    got = _ops.quantize(x, prec)
+    assert got.dtype == torch.float16
+    assert torch.equal(torch.nan_to_num(got.float(), nan=9.0), torch.nan_to_num(want.float(), nan=9.0))
+    assert torch.equal(torch.signbit(got), torch.signbit(want))
+    # ragged length (scalar tail), channels_last, through QuantizeGrad
+    assert torch.equal(_ops.quantize(x[5:1008], prec), want[5:1008])
+    g = torch.Generator().manual_seed(prec)
+    x4 = torch.randn(2, 8, 5, 5, generator=g).half().cuda().contiguous(memory_format=torch.channels_last).requires_grad_(True)
+    y4 = uf.QuantizeGrad.apply(x4, prec)
+    assert y4.dtype == torch.float16 and y4.stride() == x4.stride()
+    assert torch.equal(y4, (x4.detach() * s).round().clamp(-s + 1, s - 1) / s)
+    # a precision beyond the kernel's range takes the tensor passes
+    assert torch.equal(uf.quantize(x4.detach(), 12), (x4.detach() * 4096).round().clamp(-4095, 4095) / 4096)
