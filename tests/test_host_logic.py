@@ -96,3 +96,14 @@ def test_merged_surrogate_choice_on_the_host(monkeypatch):
     assert not ok(x, w, forward="or_2_1")                 # no fused kernel for the approximations
     monkeypatch.setenv("REXSC_MERGED_SURROGATE", "0")
     assert not ok(x, w)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path has no collectives: bench.py --gpus N > 1 exits with a message instead of printing a number."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode != 0 and "one GPU" in proc.stderr and proc.stdout.strip() == ""
